@@ -24,7 +24,7 @@ from typing import List, Optional
 import numpy as np
 import torch
 
-from ..parts.registry import PagedKV, RowState
+from ..parts.registry import PagedKV, PagedLatent, RowState
 from .allocator import NULL_PAGE, BlockAllocator, OutOfBlocks, blocks_for
 from .staging import PinnedUploader
 
@@ -59,14 +59,17 @@ class PagedGroup:
         self.covered = [0] * max_rows
         self.first_live = [0] * max_rows
         self.dirty = set()
-        self.pool_shape = (num_blocks + 1, need.n_kv_heads, block_size, need.head_dim)
+        # a latent is kept as one "head" of ``width`` elements, in one pool per slot
+        self.pool_shape = ((num_blocks + 1, 1, block_size, need.width) if isinstance(need, PagedLatent)
+                           else (num_blocks + 1, need.n_kv_heads, block_size, need.head_dim))
         self.dtype, self.device = dtype, device
         self.pools = {}
         self._upload = PinnedUploader(device) if torch.device(device).type == "cuda" else None
 
     def add_slot(self, slot_id: int):
         k = torch.zeros(self.pool_shape, dtype=self.dtype, device=self.device)
-        v = torch.zeros(self.pool_shape, dtype=self.dtype, device=self.device)
+        # (a latent serves as keys and as values: both names point at the one pool)
+        v = k if isinstance(self.need, PagedLatent) else torch.zeros(self.pool_shape, dtype=self.dtype, device=self.device)
         self.pools[slot_id] = (k, v)
 
     # -- pages a row needs / can drop ---------------------------------------------------------
@@ -149,7 +152,7 @@ class RowScalars:
 class CacheManager:
     def __init__(self, needs: List[object], max_rows: int, max_len: int, block_size: int,
                  num_blocks: int, dtype, device):
-        """needs: per cache slot a PagedKV, a RowState or None (see parts.cache_needs).
+        """needs: per cache slot a PagedKV, a PagedLatent, a RowState or None (see parts.cache_needs).
         num_blocks: usable pages of every paged group (the null page comes on top)."""
         if block_size < 1 or max_rows < 1 or max_len < 1:
             raise ValueError("block_size, max_rows and max_len must be positive")
@@ -160,7 +163,7 @@ class CacheManager:
         self._slots = []
         by_need = {}
         for slot_id, need in enumerate(needs):
-            if isinstance(need, PagedKV):
+            if isinstance(need, (PagedKV, PagedLatent)):
                 group = by_need.get(need)
                 if group is None:
                     group = PagedGroup(need, max_rows, self.table_width, block_size, num_blocks,

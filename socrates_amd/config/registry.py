@@ -11,6 +11,7 @@ from __future__ import annotations
 import json
 from pathlib import Path
 
+from .mitisun import MitisunConfig
 from .qwen3 import ConfigError, Qwen3Config
 
 _ARCHITECTURES = {}
@@ -52,16 +53,24 @@ def config_class_for(name: str):
         raise ConfigError(f"unknown architecture {name!r}; known: {known_architectures()}") from None
 
 
+def _architecture_of(raw: dict, where) -> str:
+    """The name a configuration file gives its model class: the first of ``architectures``,
+    or the string ``architecture``."""
+    archs = raw.get("architectures")
+    if archs:
+        return archs[0]
+    if isinstance(raw.get("architecture"), str):
+        return raw["architecture"]
+    raise ConfigError(f"{where} has no 'architectures' or 'architecture' entry; known: {known_architectures()}")
+
+
 def load_config(folder):
     """Read ``folder/config.json`` and return the typed configuration it names."""
     path = Path(folder) / "config.json"
     if not path.is_file():
         raise ConfigError(f"{path} not found")
     raw = json.loads(path.read_text())
-    archs = raw.get("architectures")
-    if not archs:
-        raise ConfigError(f"{path} has no 'architectures' entry; known: {known_architectures()}")
-    return config_class_for(archs[0]).from_dict(raw)
+    return config_class_for(_architecture_of(raw, path)).from_dict(raw)
 
 
 _PRESETS = Path(__file__).resolve().parent / "presets"
@@ -84,7 +93,8 @@ def load_preset(name: str):
     """The typed configuration of a preset; which class reads it is decided by its own
     ``architectures`` entry, as for a model folder."""
     raw = json.loads(preset_path(name).read_text())
-    return config_class_for(raw["architectures"][0]).from_dict(raw)
+    return config_class_for(_architecture_of(raw, name)).from_dict(raw)
 
 
 register_architecture("Qwen3ForCausalLM", Qwen3Config)
+register_architecture("Mitisun", MitisunConfig)

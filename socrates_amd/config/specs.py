@@ -88,6 +88,143 @@ class SwiGLUSpec:
 
 
 @dataclass(frozen=True)
+class ScalarRMSNormSpec:
+    """y = x / sqrt(mean(x^2) + eps) * g over the last ``dim`` elements, with one stored
+    number g for all of them (the tensor carries the norm's own name, no suffix)."""
+    dim: int
+    eps: float
+
+
+@dataclass(frozen=True)
+class PairRopeSpec:
+    """Rotary encoding in the interleaved layout: elements 2i and 2i + 1 of the first ``dims``
+    of a vector are one pair, turned by position * base ** (-2i / dims); the rest passes."""
+    dims: int
+    base: float
+
+    def __post_init__(self):
+        if self.dims < 2 or self.dims % 2:
+            raise ValueError(f"a rotation over pairs needs an even number of dimensions, not {self.dims}")
+        if not self.base > 0:
+            raise ValueError("the rotation's base must be positive")
+
+
+@dataclass(frozen=True)
+class ClampedGLUSpec:
+    """y = Wd(g * sigmoid(slope * g) * (u + 1)) with g = min(Wg x, limit) and
+    u = clamp(Wu x, -limit, limit), no bias."""
+    hidden: int
+    intermediate: int
+    limit: float
+    slope: float = 1.702
+
+    def __post_init__(self):
+        if not self.limit > 0:
+            raise ValueError("limit must be positive")
+
+
+@dataclass(frozen=True)
+class SigmoidGateSpec:
+    """sigmoid(W h + b), [dim] from [dim]: what a block multiplies a branch's result by."""
+    dim: int
+
+
+@dataclass(frozen=True)
+class WkvSpec:
+    """Time mixing with a matrix state per head and a decay per key channel that depends on
+    the token: each of r, k, v, g, w reads its own blend of the token's input and the one
+    before it; o_t = (S + diag(u) k_t v_t^T)^T r_t, S <- diag(w_t) S + k_t v_t^T with
+    w = exp(-exp(W2 tanh(W1 x_w) + w0)); each head's o over its root mean square, times a gain,
+    times silu(g), then the output projection. ``decay_rank`` 0: whatever W1 holds on disk."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    eps: float
+    decay_rank: int = 0
+
+    def __post_init__(self):
+        if self.n_heads < 1 or not 1 <= self.head_dim <= 256:
+            raise ValueError(f"wkv: {self.n_heads} heads of {self.head_dim}: head sizes run from 1 to 256")
+
+
+@dataclass(frozen=True)
+class Mamba2Spec:
+    """State-space mixing with a scalar decay per head (Mamba-2): the input projection gives
+    [z | x | B | C | dt]; x, B, C pass a causal convolution of ``conv_taps`` taps per channel
+    and silu; dt = softplus(dt + bias); S <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x
+    per head (``state`` x ``head_dim``), heads sharing B and C in ``n_groups`` groups; y times
+    silu(z), RMS-normed in ``norm_groups`` equal parts, times a gain, then the output projection."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    state: int
+    n_groups: int
+    conv_taps: int
+    norm_groups: int
+    eps: float
+
+    def __post_init__(self):
+        if self.n_heads % self.n_groups:
+            raise ValueError(f"mamba2: {self.n_heads} heads do not divide into {self.n_groups} groups")
+        if (self.n_heads * self.head_dim) % self.norm_groups:
+            raise ValueError(f"mamba2: {self.n_heads * self.head_dim} channels do not divide into {self.norm_groups} norm groups")
+        if not 1 <= self.state <= 256 or self.head_dim < 1 or self.conv_taps < 1:
+            raise ValueError(f"mamba2: state {self.state} (1 to 256), head size {self.head_dim}, {self.conv_taps} taps")
+
+    @property
+    def inner(self) -> int:
+        return self.n_heads * self.head_dim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.n_groups * self.state
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Softmax attention whose keys and values are expanded from one cached latent per token.
+
+    Queries: q = Wuq rmsnorm(Wdq h), per head [``head_dim`` plain | ``rot_dim`` rotated].
+    Keys and values: Wdkv h = [latent (``kv_rank``, RMS-normed) | one rotated key part
+    (``rot_dim``) that all heads share]; per head the plain key is Wuk latent, the value Wuv
+    latent (``v_dim``). score = scale * (q_plain . k_plain + q_rot . k_rot); a query at
+    position p sees keys p - window + 1 .. p (all up to p if ``window`` is None).
+    ``own_kv`` False: the layer has no Wdkv and reads the cache slot another layer writes.
+    ``keep``: how many positions back the cache slot has to hold (the widest window of all
+    layers that read it; None: all)."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    rot_dim: int
+    v_dim: int
+    kv_rank: int
+    q_rank: int
+    scale: float
+    position: PairRopeSpec
+    eps: float
+    window: Optional[int] = None
+    keep: Optional[int] = None
+    own_kv: bool = True
+
+    def __post_init__(self):
+        if self.position.dims > self.rot_dim:
+            raise ValueError(f"the rotation covers {self.position.dims} dimensions, the rotated part has {self.rot_dim}")
+        if self.window is not None and self.window < 1:
+            raise ValueError("window must be at least 1")
+        if self.window is None and self.keep is not None or (
+                self.window is not None and self.keep is not None and self.keep < self.window):
+            raise ValueError("the cache must keep at least the layer's own window")
+        if not 16 <= self.cache_width <= 256:
+            raise ValueError(f"latent of {self.kv_rank} + rotated part of {self.rot_dim}: the attention kernels take "
+                             "up to 256 together")
+
+    @property
+    def cache_width(self) -> int:
+        """Elements per cached token: latent and rotated key part, padded to the kernels' step."""
+        return (self.kv_rank + self.rot_dim + 15) // 16 * 16
+
+
+@dataclass(frozen=True)
 class BlockSpec:
     """One layer: which mixer, feed-forward and norms, how they are arranged,
     and the prefix its tensors carry on disk.
@@ -105,6 +242,16 @@ class BlockSpec:
         ("norm1", "input_layernorm"), ("mixer", "self_attn"),
         ("norm2", "post_attention_layernorm"), ("ffn", "mlp"))
     arrangement: str = "prenorm"
+    # For the arrangement "sandwich": x <- x + mult * post_norm(gate(h) * branch(h)) with
+    # h = norm(x), for the mixer and then for the feed-forward (``ffn`` None: the layer has
+    # none, and no norm2, post_norm2 or gate2 either); a gate of None multiplies by one.
+    post_norm1: object = None
+    post_norm2: object = None
+    gate1: object = None
+    gate2: object = None
+    residual_mult: float = 1.0
+
+    ROLES = ("norm1", "mixer", "norm2", "ffn", "post_norm1", "post_norm2", "gate1", "gate2")
 
     def name_of(self, role: str) -> str:
         return self.prefix + dict(self.names)[role]
@@ -141,6 +288,8 @@ class ModelPlan:
     # What some architectures put between the parts (none of it in the reference's model, so
     # the defaults leave the step as it is): the embedding's rows times a constant; the logits
     # times a constant, then logit_softcap * tanh(logits / logit_softcap).
+    # names a checkpoint may also hold and that are not read (tensors of a sub-part a layer lacks)
+    ignorable: Tuple[str, ...] = field(default=())
     embedding_scale: float = 1.0
     logit_scale: float = 1.0
     logit_softcap: Optional[float] = None

@@ -21,11 +21,19 @@ def register_arrangement(name: str, cls) -> None:
 def block_tensors(spec: BlockSpec):
     """{full tensor name: TensorDecl} of one layer."""
     out = {}
-    for role in ("norm1", "mixer", "norm2", "ffn"):
+    for role in spec.ROLES:
         sub = getattr(spec, role)
+        if sub is None:
+            continue
         for local, decl in tensors_of(sub).items():
-            out[f"{spec.name_of(role)}.{local}"] = decl
+            out[_joined(spec.name_of(role), local)] = decl
     return out
+
+
+def _joined(base: str, local: str) -> str:
+    """A part's tensor on disk: the part's name, a dot, the local name; a local name of ""
+    is the tensor that carries the part's own name."""
+    return f"{base}.{local}" if local else base
 
 
 def build_block(spec: BlockSpec, weights, ops):
@@ -39,8 +47,7 @@ def build_block(spec: BlockSpec, weights, ops):
 
 def _sub_tensors(spec: BlockSpec, role: str, weights):
     sub = getattr(spec, role)
-    prefix = spec.name_of(role) + "."
-    return {local: weights[prefix + local] for local in tensors_of(sub)}
+    return {local: weights[_joined(spec.name_of(role), local)] for local in tensors_of(sub)}
 
 
 class Normed:
@@ -106,4 +113,55 @@ class PreNormBlock:
         return self._branch(self.ffn, (h, ctx), residual, getattr(nxt, "norm1", None), getattr(nxt, "mixer", None))
 
 
+class SandwichBlock:
+    """x <- x + m * post_norm(gate(h) * branch(h)) with h = norm(x), for the mixer and then for
+    the feed-forward (a layer may have none). The gate is sigmoid(W h + b) on the branch's own
+    input; the residual stream stays float32. What closes a branch is one kernel: gate, the
+    norm of the branch's result, the scaled sum into the stream, and the norm that opens the
+    next branch (this block's second, or the next block's first)."""
+    chains = True
+
+    def __init__(self, spec: BlockSpec, weights, ops):
+        self.spec, self.ops = spec, ops
+        for role in spec.ROLES:
+            sub = getattr(spec, role)
+            setattr(self, role, None if sub is None else build_part(sub, _sub_tensors(spec, role, weights), ops))
+        if self.ffn is not None and (self.norm2 is None or self.post_norm2 is None):
+            raise ValueError("a feed-forward needs the norms before and after it")
+        parts = [getattr(self, role) for role in spec.ROLES]
+        self.capturable = all(getattr(p, "capturable", True) for p in parts if p is not None)
+
+    def reserve(self, n_positions):
+        for role in self.spec.ROLES:
+            part = getattr(self, role)
+            if hasattr(part, "reserve"):
+                part.reserve(n_positions)
+
+    def _close(self, residual, y, h, gate, post_norm, next_norm):
+        """Close a branch whose input was ``h`` and whose result is ``y``; returns the rows
+        the next branch reads (None if nothing follows in this stream)."""
+        ops = self.ops
+        logits = bias = None
+        if gate is not None:
+            logits, bias = ops.linear(h, gate.weight), gate.bias
+        gain, eps = post_norm.fusable()
+        follows = next_norm.fusable() if hasattr(next_norm, "fusable") else None
+        out = ops.gated_norm_add(residual, y, logits, bias, gain, eps, self.spec.residual_mult,
+                                 *(follows or (None, 0.0)))
+        if next_norm is not None and follows is None:
+            out = next_norm.add_norm(residual, None)
+        return out
+
+    def forward(self, residual, pending, ctx, slot, write=True, nxt=None):
+        h = pending.rows if isinstance(pending, Normed) else self.norm1.add_norm(residual, pending)
+        a = self.mixer.forward(h, ctx, slot, write)
+        first_of_next = getattr(nxt, "norm1", None)
+        h = self._close(residual, a, h, self.gate1, self.post_norm1, self.norm2 if self.ffn is not None else first_of_next)
+        if self.ffn is not None:
+            f = self.ffn.forward(h, ctx)
+            h = self._close(residual, f, h, self.gate2, self.post_norm2, first_of_next)
+        return None if h is None else Normed(h)
+
+
 register_arrangement("prenorm", PreNormBlock)
+register_arrangement("sandwich", SandwichBlock)

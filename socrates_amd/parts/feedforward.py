@@ -5,7 +5,7 @@ from __future__ import annotations
 
 import torch
 
-from ..config.specs import SwiGLUSpec
+from ..config.specs import ClampedGLUSpec, SigmoidGateSpec, SwiGLUSpec
 from .registry import TensorDecl, register_part
 
 
@@ -44,4 +44,38 @@ class SwiGLU:
         return self.ops.linear(act, self.w_down, allow_partial=True)
 
 
+class ClampedGLU:
+    """y = Wd(g * sigmoid(slope * g) * (u + 1)), g = min(Wg x, limit), u = clamp(Wu x, +-limit)."""
+
+    @staticmethod
+    def tensors(spec: ClampedGLUSpec):
+        return {"gate": TensorDecl((spec.intermediate, spec.hidden)),
+                "up": TensorDecl((spec.intermediate, spec.hidden)),
+                "down": TensorDecl((spec.hidden, spec.intermediate))}
+
+    def __init__(self, spec: ClampedGLUSpec, tensors, ops):
+        self.spec, self.ops = spec, ops
+        # one operand for gate and up: rows [gate | up]
+        self.w_gate_up = torch.cat([tensors["gate"], tensors["up"]], dim=0).contiguous()
+        self.w_down = tensors["down"]
+
+    def forward(self, x, ctx=None):
+        act = self.ops.glu_clamped(self.ops.linear(x, self.w_gate_up), self.spec.limit, self.spec.slope)
+        return self.ops.linear(act, self.w_down)
+
+
+class SigmoidGate:
+    """Holds W [dim, dim] and b [dim] of sigmoid(W h + b); the block computes it where it closes
+    a branch."""
+
+    @staticmethod
+    def tensors(spec: SigmoidGateSpec):
+        return {"": TensorDecl((spec.dim, spec.dim)), "b": TensorDecl((spec.dim,), "vector")}
+
+    def __init__(self, spec: SigmoidGateSpec, tensors, ops):
+        self.spec, self.weight, self.bias = spec, tensors[""], tensors["b"]
+
+
 register_part(SwiGLUSpec, SwiGLU)
+register_part(ClampedGLUSpec, ClampedGLU)
+register_part(SigmoidGateSpec, SigmoidGate)

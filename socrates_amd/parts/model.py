@@ -11,7 +11,7 @@ from __future__ import annotations
 import torch
 
 from ..config.specs import ModelPlan
-from .block import block_tensors, build_block
+from .block import _joined, block_tensors, build_block
 from .registry import TensorDecl, build_part, impl_of, tensors_of
 
 
@@ -21,7 +21,7 @@ def expected_tensors(plan: ModelPlan):
     for spec in plan.layers:
         out.update(block_tensors(spec))
     for local, decl in tensors_of(plan.final_norm).items():
-        out[f"{plan.final_norm_prefix}.{local}"] = decl
+        out[_joined(plan.final_norm_prefix, local)] = decl
     if plan.head_name is not None:
         out[plan.head_name] = TensorDecl((plan.vocab_size, plan.hidden))
     return out
@@ -48,7 +48,7 @@ class DecoderModel:
         self.plan, self.ops = plan, ops
         self.embed = weights[plan.embedding_name]
         self.blocks = [build_block(spec, weights, ops) for spec in plan.layers]
-        norm_tensors = {local: weights[f"{plan.final_norm_prefix}.{local}"]
+        norm_tensors = {local: weights[_joined(plan.final_norm_prefix, local)]
                         for local in tensors_of(plan.final_norm)}
         self.final_norm = build_part(plan.final_norm, norm_tensors, ops)
         self.head = self.embed if plan.head_name is None else weights[plan.head_name]

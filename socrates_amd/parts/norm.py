@@ -6,7 +6,9 @@ reference. Statistics are taken in float32 whatever the compute dtype.
 
 from __future__ import annotations
 
-from ..config.specs import RMSNormSpec
+import torch
+
+from ..config.specs import RMSNormSpec, ScalarRMSNormSpec
 from .registry import TensorDecl, register_part
 
 
@@ -43,4 +45,18 @@ class RMSNorm:
         return self.ops.rmsnorm(x, self.weight, self.spec.eps)
 
 
+class ScalarRMSNorm(RMSNorm):
+    """RMSNorm whose gain is one stored number (a tensor without dimensions that carries the
+    norm's own name). The kernels take a gain per element: the number is spread once here."""
+
+    @staticmethod
+    def tensors(spec: ScalarRMSNormSpec):
+        return {"": TensorDecl((), "vector")}
+
+    def __init__(self, spec: ScalarRMSNormSpec, tensors, ops):
+        self.spec, self.ops = spec, ops
+        self.weight = tensors[""].to(torch.float32).reshape(1).expand(spec.dim).contiguous()
+
+
 register_part(RMSNormSpec, RMSNorm)
+register_part(ScalarRMSNormSpec, ScalarRMSNorm)

@@ -44,9 +44,19 @@ class TensorDecl:
     kind "matrix": operand of a matrix product, kept in the compute dtype (a tensor
     stored in 32-bit floats stays 32-bit); "vector": gains and other small
     parameters, kept in float32 (lossless from bfloat16); "int": kept as int32.
+    A dimension of -1 is read off the stored tensor (``free``: its size where a tensor is
+    made up instead of read).
     """
     shape: Tuple[int, ...]
     kind: str = "matrix"
+    free: int = 16
+
+    def fits(self, stored) -> bool:
+        stored = tuple(stored)
+        return len(stored) == len(self.shape) and all(a in (-1, b) for a, b in zip(self.shape, stored))
+
+    def made_up_shape(self):
+        return tuple(self.free if s == -1 else s for s in self.shape)
 
 
 @dataclass(frozen=True)
@@ -54,6 +64,15 @@ class PagedKV:
     """A mixer that keeps keys and values of every position (or a window of them) in pages."""
     n_kv_heads: int
     head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class PagedLatent:
+    """A mixer that keeps one vector of ``width`` elements per position in pages (a latent
+    that keys and values are expanded from): one pool per cache slot. ``window``: how many
+    positions back the slot has to hold (None: all)."""
+    width: int
     window: Optional[int] = None
 
 

@@ -84,19 +84,20 @@ def _same_stored(where, a, b) -> bool:
     return ta.dtype == tb.dtype and ta.shape == tb.shape and torch.equal(ta, tb)
 
 
-def load_weights(folder, expected, compute_dtype, device, duplicates=()):
+def load_weights(folder, expected, compute_dtype, device, duplicates=(), ignorable=()):
     """Read the tensors named in ``expected`` ({name: TensorDecl}) from ``folder``.
 
     Returns {name: tensor on device}. Raises WeightError naming everything that
     does not fit. As under the reference's strict load, an ``lm_head.weight`` in
     the folder of a tied model is unexpected, unless ``duplicates`` ((stored name,
     expected name) pairs, ``ModelPlan.duplicates``) names it and it holds the very
-    values of the embedding table; it is then not read.
+    values of the embedding table; it is then not read. ``ignorable`` names may be in the
+    folder and are not read either (``ModelPlan.ignorable``).
     """
     folder = Path(folder)
     where = _files_of(folder)
     missing = [n for n in expected if n not in where]
-    unexpected = [n for n in where if n not in expected]
+    unexpected = [n for n in where if n not in expected and n not in ignorable]
     for stored, same_as in duplicates:
         if stored in unexpected and same_as in where and _same_stored(where, stored, same_as):
             unexpected.remove(stored)
@@ -111,7 +112,7 @@ def load_weights(folder, expected, compute_dtype, device, duplicates=()):
             for name, decl in items:
                 sl = sf.get_slice(name)
                 shape = tuple(sl.get_shape())
-                if shape != tuple(decl.shape):
+                if not decl.fits(shape):
                     wrong_shape.append((name, decl.shape, shape))
                 if kept_dtype(decl.kind, sl.get_dtype(), compute_dtype) is None:
                     wrong_dtype.append((name, sl.get_dtype()))

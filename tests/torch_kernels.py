@@ -160,6 +160,143 @@ class TorchKernels:
             out[t] = torch.einsum("hgn,nhd->hgd", a, v).reshape(Hq * D).to(self.dtype)
         return out
 
+    # -- what closes a branch of a block with norms on both sides ------------------------------
+    def gated_norm_add(self, residual, y, gate_logits, gate_bias, gain, eps, mult, next_gain=None, next_eps=0.0):
+        y = y.to(self.acc)
+        if gate_logits is not None:
+            y = y * torch.sigmoid(gate_logits.to(self.acc) + gate_bias.to(self.acc))
+        residual += (mult * self._norm(y, gain, eps)).to(residual.dtype)
+        if next_gain is None:
+            return None
+        return self._norm(residual, next_gain, next_eps).to(self.dtype)
+
+    def glu_clamped(self, gate_up, limit, slope):
+        ff = gate_up.shape[-1] // 2
+        g = torch.clamp(gate_up[..., :ff].to(self.acc), max=limit)
+        u = torch.clamp(gate_up[..., ff:].to(self.acc), min=-limit, max=limit)
+        return (g * torch.sigmoid(slope * g) * (u + 1)).to(self.dtype)
+
+    # -- mixers with a state per row -------------------------------------------------------------
+    @staticmethod
+    def _sequences(ctx):
+        starts = ctx.seq_qstart.cpu().tolist()
+        rows = ctx.seq_rows.cpu().tolist()
+        return [(rows[i], starts[i], starts[i + 1]) for i in range(len(rows))]
+
+    def token_shift(self, h, mu, state, offset, ctx):
+        N, d = h.shape
+        hf = h.to(self.acc)
+        prev = torch.empty_like(hf)
+        for row, lo, hi in self._sequences(ctx):
+            prev[lo] = state[row, offset:offset + d].to(self.acc)
+            prev[lo + 1:hi] = hf[lo:hi - 1]
+            state[row, offset:offset + d] = hf[hi - 1].to(state.dtype)
+        return (hf.unsqueeze(0) + (prev - hf).unsqueeze(0) * mu.to(self.acc).unsqueeze(1)).to(self.dtype)
+
+    def wkv_decay(self, t, w2, w0):
+        z = torch.tanh(t.to(self.acc)) @ w2.to(self.acc).T + w0.to(self.acc)
+        return torch.exp(-torch.exp(z)).to(torch.float32 if self.acc == torch.float32 else self.acc)
+
+    def wkv(self, r, k, v, decay, g, bonus, gain, eps, H, state, offset, ctx):
+        N, C = r.shape
+        D = C // H
+        A = self.acc
+        r, k, v, decay, g = (t.to(A).view(N, H, D) for t in (r, k, v, decay, g))
+        out = torch.empty((N, H, D), dtype=A)
+        for row, lo, hi in self._sequences(ctx):
+            S = state[row, offset:offset + H * D * D].to(A).view(H, D, D).clone()
+            for t in range(lo, hi):
+                kv = k[t].unsqueeze(-1) * v[t].unsqueeze(-2)
+                out[t] = torch.einsum("hk,hkv->hv", r[t], S + bonus.to(A).unsqueeze(-1) * kv)
+                S = decay[t].unsqueeze(-1) * S + kv
+            state[row, offset:offset + H * D * D] = S.reshape(-1).to(state.dtype)
+        out = out / torch.sqrt(out.pow(2).mean(-1, keepdim=True) + eps)
+        out = out * gain.to(A).view(H, D) * (g * torch.sigmoid(g))
+        return out.reshape(N, C).to(self.dtype)
+
+    def causal_conv_silu(self, x, col, C, weight, bias, state, offset, ctx):
+        taps = weight.shape[1]
+        A = self.acc
+        xin = x[:, col:col + C].to(A)
+        out = torch.empty((x.shape[0], C), dtype=A)
+        for row, lo, hi in self._sequences(ctx):
+            before = state[row, offset:offset + (taps - 1) * C].to(A).view(taps - 1, C)
+            seq = torch.cat([before, xin[lo:hi]], dim=0)
+            n = hi - lo
+            y = bias.to(A).expand(n, -1).clone()
+            for j in range(taps):
+                y = y + seq[j:j + n] * weight[:, j].to(A)
+            out[lo:hi] = y
+            if taps > 1:
+                state[row, offset:offset + (taps - 1) * C] = seq[n:].reshape(-1).to(state.dtype)
+        return (out * torch.sigmoid(out)).to(self.dtype)
+
+    def ssd(self, xbc, dt, dt_bias, a_log, skip, H, P, Ns, G, state, offset, ctx):
+        A = self.acc
+        N = xbc.shape[0]
+        inner = H * P
+        x = xbc[:, :inner].to(A).view(N, H, P)
+        B = xbc[:, inner:inner + G * Ns].to(A).view(N, G, Ns).repeat_interleave(H // G, dim=1)
+        Cm = xbc[:, inner + G * Ns:].to(A).view(N, G, Ns).repeat_interleave(H // G, dim=1)
+        dt = torch.nn.functional.softplus(dt.to(A) + dt_bias.to(A), threshold=30.0)
+        rate = torch.exp(a_log.to(A))
+        out = torch.empty((N, H, P), dtype=A)
+        for row, lo, hi in self._sequences(ctx):
+            S = state[row, offset:offset + H * Ns * P].to(A).view(H, Ns, P).clone()
+            for t in range(lo, hi):
+                S = torch.exp(-rate * dt[t]).view(H, 1, 1) * S + (dt[t].unsqueeze(-1) * B[t]).unsqueeze(-1) * x[t].unsqueeze(-2)
+                out[t] = torch.einsum("hn,hnp->hp", Cm[t], S) + skip.to(A).unsqueeze(-1) * x[t]
+            state[row, offset:offset + H * Ns * P] = S.reshape(-1).to(state.dtype)
+        return out.reshape(N, inner).to(torch.float32 if A == torch.float32 else A)
+
+    def gated_group_norm(self, y, z, gain, groups, eps):
+        A = self.acc
+        N, inner = y.shape
+        zz = z[:, :inner].to(A)
+        y = y.to(A) * (zz * torch.sigmoid(zz))
+        y = y.view(N, groups, inner // groups)
+        y = y / torch.sqrt(y.pow(2).mean(-1, keepdim=True) + eps)
+        return (y.reshape(N, inner) * gain.to(A)).to(self.dtype)
+
+    # -- attention over a cached latent ------------------------------------------------------------
+    def _turn_pairs(self, x, positions, inv_freq):
+        """Pairs (2i, 2i + 1) of the first 2 * len(inv_freq) elements of the last axis; x [N, ..., D]."""
+        dims = 2 * inv_freq.numel()
+        ang = positions.to(torch.float32)[:, None] * inv_freq.to(torch.float32)[None, :]
+        shape = [x.shape[0]] + [1] * (x.dim() - 2) + [dims // 2]
+        cos, sin = ang.cos().to(self.acc).view(shape), ang.sin().to(self.acc).view(shape)
+        a, b = x[..., 0:dims:2], x[..., 1:dims:2]
+        out = x.clone()
+        out[..., 0:dims:2] = a * cos - b * sin
+        out[..., 1:dims:2] = b * cos + a * sin
+        return out
+
+    def latent_write(self, kvd, R, Dr, gain, eps, inv_freq, positions, token_rows, slot):
+        A = self.acc
+        latent = self._norm(kvd[:, :R], gain, eps)
+        shared = self._turn_pairs(kvd[:, R:R + Dr].to(A), positions, inv_freq)
+        bs = slot.block_size
+        pos = positions.long()
+        page = slot.block_table[token_rows.long(), pos // bs].long()
+        row = torch.zeros((kvd.shape[0], slot.k.shape[-1]), dtype=A)
+        row[:, :R], row[:, R:R + Dr] = latent, shared
+        slot.k[page, 0, pos % bs] = row.to(slot.k.dtype)
+
+    def latent_query(self, q, H, D, Dr, w_uk_t, width, inv_freq, positions):
+        A = self.acc
+        N = q.shape[0]
+        R = w_uk_t.shape[1]
+        q = q.to(A).view(N, H, D + Dr)
+        out = torch.zeros((N, H, width), dtype=A)
+        out[..., :R] = torch.einsum("nhd,hrd->nhr", q[..., :D], w_uk_t.to(A))
+        out[..., R:R + Dr] = self._turn_pairs(q[..., D:], positions, inv_freq)
+        return out.to(self.dtype)
+
+    def head_project(self, x, w):
+        H, n_out, K = w.shape
+        y = torch.einsum("nhk,hok->nho", x[..., :K].to(self.acc), w.to(self.acc))
+        return y.reshape(x.shape[0], H * n_out).to(self.dtype)
+
     # -- sampling ----------------------------------------------------------------------------
     def argmax(self, logits):
         return logits.argmax(dim=-1).to(torch.int32)
