@@ -1,0 +1,549 @@
+// Kernels of the mixers beyond grouped-query attention, and of blocks with norms on both
+// sides of a branch: the gated close of a branch, a clamped gated activation, the blends of
+// a token with the one before it, two recurrences with a matrix state per head (decay per key
+// channel; scalar decay), a short causal convolution, a gated group norm, and what attention
+// over a cached latent needs around the paged-attention kernels (norm + rotation + page write
+// of the latent, rotation of the queries, one small product per head).
+//
+// Statistics, gates, decays, exponentials, angles and states are float32 whatever the compute
+// dtype; a value is rounded once, where it is stored in the compute dtype.
+//
+// Sequences: kernels that carry state walk the tokens of each sequence of the step in order.
+// seq_qstart [S + 1] gives each sequence's tokens among the step's, seq_rows [S] its row of
+// the state tensor [rows, stride] (float32).
+#include "common.h"
+
+__device__ __forceinline__ float soc_sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
+
+// ---- the close of a branch ---------------------------------------------------------------------
+// residual += mult * gain * g / rms(g) with g = y * sigmoid(logits + bias) (no gate: g = y);
+// then, if next_gain is given, out = residual / rms(residual) * next_gain.
+template <typename T>
+__global__ void __launch_bounds__(256)
+gated_norm_add_kernel(float* __restrict__ residual, const T* __restrict__ y, const T* __restrict__ logits,
+                      const float* __restrict__ bias, const float* __restrict__ gain, float eps, float mult,
+                      const float* __restrict__ next_gain, float next_eps, T* __restrict__ out, int d) {
+    __shared__ float scratch[16];
+    const size_t base = (size_t)blockIdx.x * d;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < d; c += blockDim.x) {
+        float g = to_float(y[base + c]);
+        if (logits) g *= soc_sigmoid(to_float(logits[base + c]) + bias[c]);
+        ss += g * g;
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = mult / sqrtf(ss / (float)d + eps);
+    float rr = 0.f;
+    for (int c = threadIdx.x; c < d; c += blockDim.x) {
+        float g = to_float(y[base + c]);
+        if (logits) g *= soc_sigmoid(to_float(logits[base + c]) + bias[c]);
+        const float r = residual[base + c] + scale * gain[c] * g;
+        residual[base + c] = r;
+        rr += r * r;
+    }
+    if (!next_gain) return;
+    rr = block_sum(rr, scratch);
+    const float inv = 1.f / sqrtf(rr / (float)d + next_eps);
+    for (int c = threadIdx.x; c < d; c += blockDim.x)
+        out[base + c] = from_float<T>(residual[base + c] * inv * next_gain[c]);
+}
+
+SOC_EXPORT int soc_gated_norm_add(float* residual, const void* y, const void* logits, const float* bias,
+                                  const float* gain, float eps, float mult, const float* next_gain, float next_eps,
+                                  void* out, int N, int d, int dtype, hipStream_t stream) {
+    if (N <= 0) return 0;
+    if (dtype == 0)
+        hipLaunchKernelGGL(gated_norm_add_kernel<float>, dim3(N), dim3(256), 0, stream, residual, (const float*)y,
+                           (const float*)logits, bias, gain, eps, mult, next_gain, next_eps, (float*)out, d);
+    else
+        hipLaunchKernelGGL(gated_norm_add_kernel<bf16>, dim3(N), dim3(256), 0, stream, residual, (const bf16*)y,
+                           (const bf16*)logits, bias, gain, eps, mult, next_gain, next_eps, (bf16*)out, d);
+    return soc_last_error();
+}
+
+// ---- g * sigmoid(slope g) * (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit) ---------
+template <typename T>
+__global__ void glu_clamped_kernel(const T* __restrict__ gate_up, T* __restrict__ out, size_t total, int ff,
+                                   float limit, float slope) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const size_t n = i / ff, c = i % ff;
+    const float g = fminf(to_float(gate_up[n * 2 * ff + c]), limit);
+    const float u = fminf(fmaxf(to_float(gate_up[n * 2 * ff + ff + c]), -limit), limit);
+    out[i] = from_float<T>(g * soc_sigmoid(slope * g) * (u + 1.f));
+}
+
+SOC_EXPORT int soc_glu_clamped(const void* gate_up, void* out, int N, int ff, float limit, float slope, int dtype,
+                               hipStream_t stream) {
+    const size_t total = (size_t)N * ff;
+    if (total == 0) return 0;
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (dtype == 0)
+        hipLaunchKernelGGL(glu_clamped_kernel<float>, grid, dim3(256), 0, stream, (const float*)gate_up, (float*)out,
+                           total, ff, limit, slope);
+    else
+        hipLaunchKernelGGL(glu_clamped_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)gate_up, (bf16*)out,
+                           total, ff, limit, slope);
+    return soc_last_error();
+}
+
+// ---- blends of a token's input with the one before it ---------------------------------------------
+// out[s, n, c] = h[n, c] + (prev[n, c] - h[n, c]) * mu[s, c]; prev of a sequence's first token of
+// the step is what the row's state holds, which then becomes the input of its last token. Grid
+// (chunks of SHIFT_CHUNK tokens, sequences): the workgroup of a sequence's first chunk is the
+// only one that touches the state, each thread its own columns, reading before writing.
+constexpr int SHIFT_CHUNK = 8;
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+token_shift_kernel(const T* __restrict__ h, const float* __restrict__ mu, int n_streams, float* __restrict__ state,
+                   size_t stride, int offset, const int* __restrict__ seq_qstart, const int* __restrict__ seq_rows,
+                   T* __restrict__ out, int N, int d) {
+    const int seq = blockIdx.y;
+    const int lo = seq_qstart[seq], hi = seq_qstart[seq + 1];
+    const int first = lo + blockIdx.x * SHIFT_CHUNK;
+    if (first >= hi) return;
+    const int last = min(first + SHIFT_CHUNK, hi);
+    float* kept = state + (size_t)seq_rows[seq] * stride + offset;
+    for (int c = threadIdx.x; c < d; c += blockDim.x) {
+        float prev = first == lo ? kept[c] : to_float(h[(size_t)(first - 1) * d + c]);
+        for (int n = first; n < last; ++n) {
+            const float cur = to_float(h[(size_t)n * d + c]);
+            const float diff = prev - cur;
+            for (int s = 0; s < n_streams; ++s)
+                out[((size_t)s * N + n) * d + c] = from_float<T>(cur + diff * mu[(size_t)s * d + c]);
+            prev = cur;
+        }
+        if (first == lo) kept[c] = to_float(h[(size_t)(hi - 1) * d + c]);
+    }
+}
+
+SOC_EXPORT int soc_token_shift(const void* h, const float* mu, int n_streams, float* state, long long stride, int offset,
+                               const int* seq_qstart, const int* seq_rows, void* out, int N, int d, int n_seqs,
+                               int max_q_len, int dtype, hipStream_t stream) {
+    if (N <= 0 || n_seqs <= 0) return 0;
+    const dim3 grid((max_q_len + SHIFT_CHUNK - 1) / SHIFT_CHUNK, n_seqs);
+    if (dtype == 0)
+        hipLaunchKernelGGL(token_shift_kernel<float>, grid, dim3(256), 0, stream, (const float*)h, mu, n_streams, state,
+                           (size_t)stride, offset, seq_qstart, seq_rows, (float*)out, N, d);
+    else
+        hipLaunchKernelGGL(token_shift_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)h, mu, n_streams, state,
+                           (size_t)stride, offset, seq_qstart, seq_rows, (bf16*)out, N, d);
+    return soc_last_error();
+}
+
+// ---- decay = exp(-exp(tanh(t) W2^T + w0)) --------------------------------------------------------
+// t [N, rank] float32; W2 [C, rank]; one workgroup per token keeps tanh(t) in LDS.
+template <typename T>
+__global__ void __launch_bounds__(256)
+wkv_decay_kernel(const float* __restrict__ t, const T* __restrict__ w2, const float* __restrict__ w0,
+                 float* __restrict__ out, int C, int rank) {
+    extern __shared__ float th[];
+    const int n = blockIdx.x;
+    for (int j = threadIdx.x; j < rank; j += blockDim.x) th[j] = tanhf(t[(size_t)n * rank + j]);
+    __syncthreads();
+    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+        float z = 0.f;
+        const T* row = w2 + (size_t)c * rank;
+        for (int j = 0; j < rank; ++j) z = fmaf(th[j], to_float(row[j]), z);
+        out[(size_t)n * C + c] = expf(-expf(z + w0[c]));
+    }
+}
+
+SOC_EXPORT int soc_wkv_decay(const float* t, const void* w2, const float* w0, float* out, int N, int C, int rank,
+                             int dtype, hipStream_t stream) {
+    if (N <= 0) return 0;
+    const size_t lds = (size_t)rank * sizeof(float);
+    if (dtype == 0)
+        hipLaunchKernelGGL(wkv_decay_kernel<float>, dim3(N), dim3(256), lds, stream, t, (const float*)w2, w0, out, C, rank);
+    else
+        hipLaunchKernelGGL(wkv_decay_kernel<bf16>, dim3(N), dim3(256), lds, stream, t, (const bf16*)w2, w0, out, C, rank);
+    return soc_last_error();
+}
+
+// ---- recurrence with a decay per key channel -------------------------------------------------------
+// Per (head, sequence): thread j owns column j of the state S [D keys, D values] in registers.
+// o_t[j] = sum_i r_t[i] (S[i, j] + u[i] k_t[i] v_t[j]); S[i, j] <- w_t[i] S[i, j] + k_t[i] v_t[j].
+// Then o over its root mean square over the head, times gain, times silu(g).
+template <typename T, int DK>
+__global__ void __launch_bounds__(256)
+wkv_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ decay,
+           const T* __restrict__ g, const float* __restrict__ bonus, const float* __restrict__ gain, float eps,
+           int H, int D, float* __restrict__ state, size_t stride, int offset, const int* __restrict__ seq_qstart,
+           const int* __restrict__ seq_rows, T* __restrict__ out) {
+    __shared__ float sr[DK], sk[DK], sw[DK], su[DK], scratch[16];
+    const int head = blockIdx.x, seq = blockIdx.y, j = threadIdx.x;
+    const int lo = seq_qstart[seq], hi = seq_qstart[seq + 1];
+    if (lo >= hi) return;
+    const bool live = j < D;
+    float* S = state + (size_t)seq_rows[seq] * stride + offset + (size_t)head * D * D;
+    float s[DK];
+#pragma unroll
+    for (int i = 0; i < DK; ++i) s[i] = (live && i < D) ? S[(size_t)i * D + j] : 0.f;
+    if (j < DK) su[j] = live ? bonus[head * D + j] : 0.f;
+    const size_t C = (size_t)H * D;
+    for (int n = lo; n < hi; ++n) {
+        const size_t at = (size_t)n * C + (size_t)head * D + j;
+        __syncthreads();
+        if (j < DK) {
+            sr[j] = live ? to_float(r[at]) : 0.f;
+            sk[j] = live ? to_float(k[at]) : 0.f;
+            sw[j] = live ? decay[at] : 0.f;
+        }
+        __syncthreads();
+        const float vj = live ? to_float(v[at]) : 0.f;
+        float o = 0.f;
+#pragma unroll
+        for (int i = 0; i < DK; ++i) {
+            const float kv = sk[i] * vj;
+            o = fmaf(sr[i], fmaf(su[i], kv, s[i]), o);
+            s[i] = fmaf(sw[i], s[i], kv);
+        }
+        const float ss = block_sum(live ? o * o : 0.f, scratch);
+        if (live) {
+            const float gate = to_float(g[at]);
+            out[at] = from_float<T>(o / sqrtf(ss / (float)D + eps) * gain[head * D + j] * gate * soc_sigmoid(gate));
+        }
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < DK; ++i)
+            if (i < D) S[(size_t)i * D + j] = s[i];
+    }
+}
+
+template <typename T, int DK>
+static void launch_wkv(const void* r, const void* k, const void* v, const float* decay, const void* g, const float* bonus,
+                       const float* gain, float eps, int H, int D, float* state, long long stride, int offset,
+                       const int* seq_qstart, const int* seq_rows, void* out, int n_seqs, hipStream_t stream) {
+    const int threads = (max(D, DK) + 63) / 64 * 64;
+    hipLaunchKernelGGL((wkv_kernel<T, DK>), dim3(H, n_seqs), dim3(threads), 0, stream, (const T*)r, (const T*)k,
+                       (const T*)v, decay, (const T*)g, bonus, gain, eps, H, D, state, (size_t)stride, offset, seq_qstart,
+                       seq_rows, (T*)out);
+}
+
+#define SOC_BY_STATE_SIZE(D, CALL)                                         \
+    switch (((D) + 15) / 16) {                                              \
+        case 1: CALL(16); break;   case 2: CALL(32); break;                 \
+        case 3: CALL(48); break;   case 4: CALL(64); break;                 \
+        case 5: CALL(80); break;   case 6: CALL(96); break;                 \
+        case 7: CALL(112); break;  case 8: CALL(128); break;                \
+        case 9: case 10: CALL(160); break;                                  \
+        case 11: case 12: CALL(192); break;                                 \
+        case 13: case 14: CALL(224); break;                                 \
+        case 15: case 16: CALL(256); break;                                 \
+        default: return (int)hipErrorInvalidValue;                          \
+    }
+
+SOC_EXPORT int soc_wkv(const void* r, const void* k, const void* v, const float* decay, const void* g, const float* bonus,
+                       const float* gain, float eps, int H, int D, float* state, long long stride, int offset,
+                       const int* seq_qstart, const int* seq_rows, void* out, int n_seqs, int dtype, hipStream_t stream) {
+    if (n_seqs <= 0 || H <= 0) return 0;
+    if (D < 1 || D > 256) return (int)hipErrorInvalidValue;
+#define SOC_WKV_F32(DK) launch_wkv<float, DK>(r, k, v, decay, g, bonus, gain, eps, H, D, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, stream)
+#define SOC_WKV_BF16(DK) launch_wkv<bf16, DK>(r, k, v, decay, g, bonus, gain, eps, H, D, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, stream)
+    if (dtype == 0) { SOC_BY_STATE_SIZE(D, SOC_WKV_F32) } else { SOC_BY_STATE_SIZE(D, SOC_WKV_BF16) }
+    return soc_last_error();
+}
+
+// ---- causal convolution per channel, then silu -------------------------------------------------------
+// y[n, c] = silu(bias[c] + sum_j w[c, j] in(n - (taps - 1) + j)); inputs before the step's first token
+// come from the row's state [taps - 1, C], which then becomes the step's last taps - 1 inputs.
+// Grid (channel blocks, chunks of CONV_CHUNK tokens, sequences); only a sequence's first chunk
+// touches the state (taps - 1 <= CONV_CHUNK), each thread its own channel, reading before writing.
+constexpr int CONV_CHUNK = 32;
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+causal_conv_silu_kernel(const T* __restrict__ x, int ldx, int col, int C, const float* __restrict__ w,
+                        const float* __restrict__ bias, int taps, float* __restrict__ state, size_t stride, int offset,
+                        const int* __restrict__ seq_qstart, const int* __restrict__ seq_rows, T* __restrict__ out) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    const int seq = blockIdx.z;
+    const int lo = seq_qstart[seq], hi = seq_qstart[seq + 1];
+    const int first = lo + blockIdx.y * CONV_CHUNK;
+    if (c >= C || first >= hi) return;
+    const int last = min(first + CONV_CHUNK, hi);
+    float* kept = state + (size_t)seq_rows[seq] * stride + offset;
+    const int back = taps - 1;
+    for (int n = first; n < last; ++n) {
+        float y = bias[c];
+        for (int j = 0; j < taps; ++j) {
+            const int idx = n - lo - back + j;          // among the step's tokens of this sequence
+            const float in = idx >= 0 ? to_float(x[(size_t)(lo + idx) * ldx + col + c])
+                                      : kept[(size_t)(back + idx) * C + c];
+            y = fmaf(w[(size_t)c * taps + j], in, y);
+        }
+        out[(size_t)n * C + c] = from_float<T>(y * soc_sigmoid(y));
+    }
+    if (first == lo) {
+        const int len = hi - lo;
+        for (int j = 0; j < back; ++j) {                // ascending: entry j + len is read before it is written
+            const int idx = len - back + j;
+            kept[(size_t)j * C + c] = idx >= 0 ? to_float(x[(size_t)(lo + idx) * ldx + col + c])
+                                               : kept[(size_t)(j + len) * C + c];
+        }
+    }
+}
+
+SOC_EXPORT int soc_causal_conv_silu(const void* x, int ldx, int col, int C, const float* w, const float* bias, int taps,
+                                    float* state, long long stride, int offset, const int* seq_qstart,
+                                    const int* seq_rows, void* out, int n_seqs, int max_q_len, int dtype,
+                                    hipStream_t stream) {
+    if (n_seqs <= 0 || C <= 0) return 0;
+    if (taps < 1 || taps - 1 > CONV_CHUNK) return (int)hipErrorInvalidValue;
+    const dim3 grid((C + 255) / 256, (max_q_len + CONV_CHUNK - 1) / CONV_CHUNK, n_seqs);
+    if (dtype == 0)
+        hipLaunchKernelGGL(causal_conv_silu_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, ldx, col, C, w, bias,
+                           taps, state, (size_t)stride, offset, seq_qstart, seq_rows, (float*)out);
+    else
+        hipLaunchKernelGGL(causal_conv_silu_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)x, ldx, col, C, w, bias,
+                           taps, state, (size_t)stride, offset, seq_qstart, seq_rows, (bf16*)out);
+    return soc_last_error();
+}
+
+// ---- recurrence with a scalar decay per head -------------------------------------------------------------
+// xbc [N, x (H P) | B (G Ns) | C (G Ns)]; dt = softplus(dt_raw + bias). Per (head, sequence): thread p
+// owns column p of S [Ns, P]: S[i, p] <- exp(-exp(a_log) dt) S[i, p] + dt B[i] x[p];
+// y[p] = sum_i C[i] S[i, p] + skip x[p], float32.
+template <typename T, int NK>
+__global__ void __launch_bounds__(256)
+ssd_kernel(const T* __restrict__ xbc, const float* __restrict__ dt_raw, const float* __restrict__ dt_bias,
+           const float* __restrict__ a_log, const float* __restrict__ skip, int H, int P, int Ns, int G,
+           float* __restrict__ state, size_t stride, int offset, const int* __restrict__ seq_qstart,
+           const int* __restrict__ seq_rows, float* __restrict__ out) {
+    __shared__ float sb[NK], sc[NK];
+    const int head = blockIdx.x, seq = blockIdx.y, p = threadIdx.x;
+    const int lo = seq_qstart[seq], hi = seq_qstart[seq + 1];
+    if (lo >= hi) return;
+    const bool live = p < P;
+    const int group = head / (H / G);
+    const int inner = H * P, ld = inner + 2 * G * Ns;
+    float* S = state + (size_t)seq_rows[seq] * stride + offset + (size_t)head * Ns * P;
+    float s[NK];
+#pragma unroll
+    for (int i = 0; i < NK; ++i) s[i] = (live && i < Ns) ? S[(size_t)i * P + p] : 0.f;
+    const float rate = expf(a_log[head]), through = skip[head], shift = dt_bias[head];
+    for (int n = lo; n < hi; ++n) {
+        const float z = dt_raw[(size_t)n * H + head] + shift;
+        const float dt = z > 20.f ? z : log1pf(expf(z));
+        const float keep = expf(-rate * dt);
+        const T* row = xbc + (size_t)n * ld;
+        __syncthreads();
+        if (p < NK) {
+            const bool in = p < Ns;
+            sb[p] = in ? dt * to_float(row[inner + group * Ns + p]) : 0.f;
+            sc[p] = in ? to_float(row[inner + G * Ns + group * Ns + p]) : 0.f;
+        }
+        __syncthreads();
+        const float xp = live ? to_float(row[head * P + p]) : 0.f;
+        float y = through * xp;
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            s[i] = fmaf(keep, s[i], sb[i] * xp);
+            y = fmaf(sc[i], s[i], y);
+        }
+        if (live) out[(size_t)n * inner + head * P + p] = y;
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < NK; ++i)
+            if (i < Ns) S[(size_t)i * P + p] = s[i];
+    }
+}
+
+template <typename T, int NK>
+static void launch_ssd(const void* xbc, const float* dt_raw, const float* dt_bias, const float* a_log, const float* skip,
+                       int H, int P, int Ns, int G, float* state, long long stride, int offset, const int* seq_qstart,
+                       const int* seq_rows, float* out, int n_seqs, hipStream_t stream) {
+    const int threads = (max(P, NK) + 63) / 64 * 64;
+    hipLaunchKernelGGL((ssd_kernel<T, NK>), dim3(H, n_seqs), dim3(threads), 0, stream, (const T*)xbc, dt_raw, dt_bias, a_log,
+                       skip, H, P, Ns, G, state, (size_t)stride, offset, seq_qstart, seq_rows, out);
+}
+
+SOC_EXPORT int soc_ssd(const void* xbc, const float* dt_raw, const float* dt_bias, const float* a_log, const float* skip,
+                       int H, int P, int Ns, int G, float* state, long long stride, int offset, const int* seq_qstart,
+                       const int* seq_rows, float* out, int n_seqs, int dtype, hipStream_t stream) {
+    if (n_seqs <= 0 || H <= 0) return 0;
+    if (Ns < 1 || Ns > 256 || P < 1 || P > 256 || G < 1 || H % G) return (int)hipErrorInvalidValue;
+#define SOC_SSD_F32(NK) launch_ssd<float, NK>(xbc, dt_raw, dt_bias, a_log, skip, H, P, Ns, G, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, stream)
+#define SOC_SSD_BF16(NK) launch_ssd<bf16, NK>(xbc, dt_raw, dt_bias, a_log, skip, H, P, Ns, G, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, stream)
+    if (dtype == 0) { SOC_BY_STATE_SIZE(Ns, SOC_SSD_F32) } else { SOC_BY_STATE_SIZE(Ns, SOC_SSD_BF16) }
+    return soc_last_error();
+}
+
+// ---- y * silu(z), then RMS norm in equal parts, times gain ------------------------------------------------
+// y float32 [N, inner]; z the first `inner` columns of rows of ldz elements. One workgroup per (part, token).
+template <typename T>
+__global__ void __launch_bounds__(256)
+gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, int ldz, const float* __restrict__ gain,
+                        int inner, int part, float eps, T* __restrict__ out) {
+    __shared__ float scratch[16];
+    const int n = blockIdx.y, c0 = blockIdx.x * part;
+    float ss = 0.f;
+    for (int c = c0 + threadIdx.x; c < c0 + part; c += blockDim.x) {
+        const float zz = to_float(z[(size_t)n * ldz + c]);
+        const float v = y[(size_t)n * inner + c] * zz * soc_sigmoid(zz);
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.f / sqrtf(ss / (float)part + eps);
+    for (int c = c0 + threadIdx.x; c < c0 + part; c += blockDim.x) {
+        const float zz = to_float(z[(size_t)n * ldz + c]);
+        const float v = y[(size_t)n * inner + c] * zz * soc_sigmoid(zz);
+        out[(size_t)n * inner + c] = from_float<T>(v * inv * gain[c]);
+    }
+}
+
+SOC_EXPORT int soc_gated_group_norm(const float* y, const void* z, int ldz, const float* gain, int N, int inner, int parts,
+                                    float eps, void* out, int dtype, hipStream_t stream) {
+    if (N <= 0) return 0;
+    if (parts < 1 || inner % parts) return (int)hipErrorInvalidValue;
+    const dim3 grid(parts, N);
+    if (dtype == 0)
+        hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, dim3(256), 0, stream, y, (const float*)z, ldz, gain, inner,
+                           inner / parts, eps, (float*)out);
+    else
+        hipLaunchKernelGGL(gated_group_norm_kernel<bf16>, grid, dim3(256), 0, stream, y, (const bf16*)z, ldz, gain, inner,
+                           inner / parts, eps, (bf16*)out);
+    return soc_last_error();
+}
+
+// ---- a token's latent into its page ---------------------------------------------------------------------------
+// kvd [N, R + Dr]: the first R RMS-normed with gain, the rest turned pair by pair (pairs 2i, 2i + 1 of the
+// first 2 * half by position * inv_freq[i]); both go to the token's place in the pool
+// [pages, 1, block, width], the padding up to width as zeros. One wave per token.
+template <typename T>
+__global__ void __launch_bounds__(64)
+latent_write_kernel(const T* __restrict__ kvd, int R, int Dr, const float* __restrict__ gain, float eps,
+                    const float* __restrict__ inv_freq, int half, const int* __restrict__ positions,
+                    const int* __restrict__ token_rows, const int* __restrict__ table, int table_width,
+                    T* __restrict__ pool, int block, int width) {
+    const int n = blockIdx.x, lane = threadIdx.x;
+    const T* row = kvd + (size_t)n * (R + Dr);
+    const int pos = positions[n];
+    const int page = table[(size_t)token_rows[n] * table_width + pos / block];
+    T* dst = pool + ((size_t)page * block + pos % block) * width;
+    float ss = 0.f;
+    for (int c = lane; c < R; c += 64) { const float v = to_float(row[c]); ss += v * v; }
+    ss = wave_sum(ss);
+    const float inv = 1.f / sqrtf(ss / (float)R + eps);
+    for (int c = lane; c < R; c += 64) dst[c] = from_float<T>(to_float(row[c]) * inv * gain[c]);
+    for (int i = lane; i < Dr / 2; i += 64) {
+        const float a = to_float(row[R + 2 * i]), b = to_float(row[R + 2 * i + 1]);
+        if (i < half) {
+            float sn, cs;
+            sincosf((float)pos * inv_freq[i], &sn, &cs);
+            dst[R + 2 * i] = from_float<T>(a * cs - b * sn);
+            dst[R + 2 * i + 1] = from_float<T>(b * cs + a * sn);
+        } else {
+            dst[R + 2 * i] = from_float<T>(a);
+            dst[R + 2 * i + 1] = from_float<T>(b);
+        }
+    }
+    if (lane == 0 && (Dr & 1)) dst[R + Dr - 1] = row[R + Dr - 1];
+    for (int c = R + Dr + lane; c < width; c += 64) dst[c] = from_float<T>(0.f);
+}
+
+SOC_EXPORT int soc_latent_write(const void* kvd, int N, int R, int Dr, const float* gain, float eps, const float* inv_freq,
+                                int half, const int* positions, const int* token_rows, const int* table, int table_width,
+                                void* pool, int block, int width, int dtype, hipStream_t stream) {
+    if (N <= 0) return 0;
+    if (2 * half > Dr || R + Dr > width) return (int)hipErrorInvalidValue;
+    if (dtype == 0)
+        hipLaunchKernelGGL(latent_write_kernel<float>, dim3(N), dim3(64), 0, stream, (const float*)kvd, R, Dr, gain, eps, inv_freq,
+                           half, positions, token_rows, table, table_width, (float*)pool, block, width);
+    else
+        hipLaunchKernelGGL(latent_write_kernel<bf16>, dim3(N), dim3(64), 0, stream, (const bf16*)kvd, R, Dr, gain, eps, inv_freq,
+                           half, positions, token_rows, table, table_width, (bf16*)pool, block, width);
+    return soc_last_error();
+}
+
+// ---- the rotated part of every head's query, beside the folded plain part ---------------------------------------
+// q [N, H, D + Dr] -> out [N, H, width]: out[.., R : R + Dr] = turned q[.., D :], zeros behind it.
+// (out[.., : R] is written by the product per head.) One thread per (token, head, pair or padding element).
+template <typename T>
+__global__ void latent_query_turn_kernel(const T* __restrict__ q, int H, int D, int Dr, int R, int width,
+                                         const float* __restrict__ inv_freq, int half, const int* __restrict__ positions,
+                                         T* __restrict__ out, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int per = width - R;                      // elements behind the folded part
+    const int e = (int)(i % per);
+    const size_t nh = i / per;
+    const int n = (int)(nh / H);
+    const T* src = q + nh * (D + Dr) + D;
+    T* dst = out + nh * width + R;
+    if (e >= Dr) { dst[e] = from_float<T>(0.f); return; }
+    const int pair = e / 2;
+    if (pair >= half || (e | 1) >= Dr) { dst[e] = src[e]; return; }
+    float sn, cs;
+    sincosf((float)positions[n] * inv_freq[pair], &sn, &cs);
+    const float a = to_float(src[2 * pair]), b = to_float(src[2 * pair + 1]);
+    dst[e] = from_float<T>((e & 1) ? b * cs + a * sn : a * cs - b * sn);
+}
+
+SOC_EXPORT int soc_latent_query_turn(const void* q, int N, int H, int D, int Dr, int R, int width, const float* inv_freq,
+                                     int half, const int* positions, void* out, int dtype, hipStream_t stream) {
+    const size_t total = (size_t)N * H * (width - R);
+    if (total == 0) return 0;
+    if (2 * half > Dr || R + Dr > width) return (int)hipErrorInvalidValue;
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (dtype == 0)
+        hipLaunchKernelGGL(latent_query_turn_kernel<float>, grid, dim3(256), 0, stream, (const float*)q, H, D, Dr, R, width,
+                           inv_freq, half, positions, (float*)out, total);
+    else
+        hipLaunchKernelGGL(latent_query_turn_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)q, H, D, Dr, R, width,
+                           inv_freq, half, positions, (bf16*)out, total);
+    return soc_last_error();
+}
+
+// ---- one small product per head ------------------------------------------------------------------------------------
+// out[n, h, o] = sum_k x[n, h, k] w[h, o, k], k < K, o < n_out; x rows of ldx elements per head (its first K are
+// read), out rows of ldo elements per head (its first n_out are written). Tiles of 16 tokens x 64 outputs,
+// 32 k at a time through LDS; float32 sums, k in order.
+template <typename T>
+__global__ void __launch_bounds__(256)
+head_linear_kernel(const T* __restrict__ x, int ldx, const T* __restrict__ w, T* __restrict__ out, int ldo,
+                   int N, int H, int n_out, int K) {
+    __shared__ float xs[16][33], ws[64][33];
+    const int head = blockIdx.z, n0 = blockIdx.y * 16, o0 = blockIdx.x * 64;
+    const int to = threadIdx.x % 64, tn = threadIdx.x / 64;          // output column; token group of 4
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        for (int e = threadIdx.x; e < 16 * 32; e += 256) {
+            const int rn = e / 32, rk = e % 32;
+            xs[rn][rk] = (n0 + rn < N && k0 + rk < K) ? to_float(x[((size_t)(n0 + rn) * H + head) * ldx + k0 + rk]) : 0.f;
+        }
+        for (int e = threadIdx.x; e < 64 * 32; e += 256) {
+            const int ro = e / 32, rk = e % 32;
+            ws[ro][rk] = (o0 + ro < n_out && k0 + rk < K) ? to_float(w[((size_t)head * n_out + o0 + ro) * K + k0 + rk]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 32; ++kk) {
+            const float wv = ws[to][kk];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acc[t] = fmaf(xs[tn * 4 + t][kk], wv, acc[t]);
+        }
+        __syncthreads();
+    }
+    if (o0 + to < n_out)
+        for (int t = 0; t < 4; ++t)
+            if (n0 + tn * 4 + t < N)
+                out[((size_t)(n0 + tn * 4 + t) * H + head) * ldo + o0 + to] = from_float<T>(acc[t]);
+}
+
+SOC_EXPORT int soc_head_linear(const void* x, int ldx, const void* w, void* out, int ldo, int N, int H, int n_out, int K,
+                               int dtype, hipStream_t stream) {
+    if (N <= 0 || H <= 0 || n_out <= 0) return 0;
+    if (K < 1 || K > ldx || n_out > ldo || H > 65535 || (N + 15) / 16 > 65535) return (int)hipErrorInvalidValue;
+    const dim3 grid((n_out + 63) / 64, (N + 15) / 16, H);
+    if (dtype == 0)
+        hipLaunchKernelGGL(head_linear_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, ldx, (const float*)w,
+                           (float*)out, ldo, N, H, n_out, K);
+    else
+        hipLaunchKernelGGL(head_linear_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)x, ldx, (const bf16*)w,
+                           (bf16*)out, ldo, N, H, n_out, K);
+    return soc_last_error();
+}

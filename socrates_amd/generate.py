@@ -75,7 +75,7 @@ def main(argv=None) -> int:
         from .config import config_class_for
         from .weights import write_random_model
         raw = json.loads(open(args.random_weights).read())
-        config = config_class_for(raw["architectures"][0]).from_dict(raw)
+        config = config_class_for((raw.get("architectures") or [raw.get("architecture")])[0]).from_dict(raw)
         write_random_model(args.model, config, args.seed)
     tok = None
     if args.tokenizer:

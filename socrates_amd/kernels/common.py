@@ -50,6 +50,20 @@ _GEMM_SIGNATURES = {
     "soc_gemm_bf16_stream": [P, P, P, I, I, I, I, I, I, I, I, P],
     "soc_gemm_stream_plan": [I, I, I, I, P, P],
 }
+L = c_longlong
+_MIXER_SIGNATURES = {
+    "soc_gated_norm_add": [P, P, P, P, P, F, F, P, F, P, I, I, I, P],
+    "soc_glu_clamped": [P, P, I, I, F, F, I, P],
+    "soc_token_shift": [P, P, I, P, L, I, P, P, P, I, I, I, I, I, P],
+    "soc_wkv_decay": [P, P, P, P, I, I, I, I, P],
+    "soc_wkv": [P, P, P, P, P, P, P, F, I, I, P, L, I, P, P, P, I, I, P],
+    "soc_causal_conv_silu": [P, I, I, I, P, P, I, P, L, I, P, P, P, I, I, I, P],
+    "soc_ssd": [P, P, P, P, P, I, I, I, I, P, L, I, P, P, P, I, I, P],
+    "soc_gated_group_norm": [P, P, I, P, I, I, I, F, P, I, P],
+    "soc_latent_write": [P, I, I, I, P, F, P, I, P, P, P, I, P, I, I, I, P],
+    "soc_latent_query_turn": [P, I, I, I, I, I, I, P, I, P, P, I, P],
+    "soc_head_linear": [P, I, P, P, I, I, I, I, I, I, P],
+}
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P, P, P, I, I, I, P]}
 _ATTENTION_SIGNATURES = {
     "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, F, P, P, P],

@@ -53,7 +53,7 @@ def make_runner(folder, ops, max_rows=4, max_len=512, block_size=16, num_blocks=
     from socrates_amd.config import load_config
     config = load_config(folder)
     plan = config.plan()
-    weights = load_weights(folder, expected_tensors(plan), ops.dtype, ops.device)
+    weights = load_weights(folder, expected_tensors(plan), ops.dtype, ops.device, plan.duplicates, plan.ignorable)
     model = DecoderModel(plan, weights, ops)
     if num_blocks is None:
         num_blocks = max_rows * ((max_len + block_size - 1) // block_size)

@@ -202,7 +202,7 @@ class TorchKernels:
         D = C // H
         A = self.acc
         r, k, v, decay, g = (t.to(A).view(N, H, D) for t in (r, k, v, decay, g))
-        out = torch.empty((N, H, D), dtype=A)
+        out = torch.empty((N, H, D), dtype=A, device=r.device)
         for row, lo, hi in self._sequences(ctx):
             S = state[row, offset:offset + H * D * D].to(A).view(H, D, D).clone()
             for t in range(lo, hi):
@@ -218,7 +218,7 @@ class TorchKernels:
         taps = weight.shape[1]
         A = self.acc
         xin = x[:, col:col + C].to(A)
-        out = torch.empty((x.shape[0], C), dtype=A)
+        out = torch.empty((x.shape[0], C), dtype=A, device=x.device)
         for row, lo, hi in self._sequences(ctx):
             before = state[row, offset:offset + (taps - 1) * C].to(A).view(taps - 1, C)
             seq = torch.cat([before, xin[lo:hi]], dim=0)
@@ -240,7 +240,7 @@ class TorchKernels:
         Cm = xbc[:, inner + G * Ns:].to(A).view(N, G, Ns).repeat_interleave(H // G, dim=1)
         dt = torch.nn.functional.softplus(dt.to(A) + dt_bias.to(A), threshold=30.0)
         rate = torch.exp(a_log.to(A))
-        out = torch.empty((N, H, P), dtype=A)
+        out = torch.empty((N, H, P), dtype=A, device=xbc.device)
         for row, lo, hi in self._sequences(ctx):
             S = state[row, offset:offset + H * Ns * P].to(A).view(H, Ns, P).clone()
             for t in range(lo, hi):
@@ -278,7 +278,7 @@ class TorchKernels:
         bs = slot.block_size
         pos = positions.long()
         page = slot.block_table[token_rows.long(), pos // bs].long()
-        row = torch.zeros((kvd.shape[0], slot.k.shape[-1]), dtype=A)
+        row = torch.zeros((kvd.shape[0], slot.k.shape[-1]), dtype=A, device=kvd.device)
         row[:, :R], row[:, R:R + Dr] = latent, shared
         slot.k[page, 0, pos % bs] = row.to(slot.k.dtype)
 
@@ -287,7 +287,7 @@ class TorchKernels:
         N = q.shape[0]
         R = w_uk_t.shape[1]
         q = q.to(A).view(N, H, D + Dr)
-        out = torch.zeros((N, H, width), dtype=A)
+        out = torch.zeros((N, H, width), dtype=A, device=q.device)
         out[..., :R] = torch.einsum("nhd,hrd->nhr", q[..., :D], w_uk_t.to(A))
         out[..., R:R + Dr] = self._turn_pairs(q[..., D:], positions, inv_freq)
         return out.to(self.dtype)
