@@ -132,12 +132,19 @@ def oracle(folder, prompts):
 
 
 def compare(got, want, tol, what=""):
-    """Logits with their mean taken off (a shift of all logits changes no choice), by rows."""
+    """Logits with their mean taken off (a shift of all logits changes no choice), by rows, in units of
+    the row's spread. ``tol``: a limit for every row, or (limit for every row, limit that nine rows in
+    ten keep): rounding to bfloat16 moves a row here and there by several times the typical error,
+    a fault of a window, a state or a page moves most rows by far more."""
     got, want = got.double(), want.double()
     d = (got - got.mean(-1, keepdim=True)) - (want - want.mean(-1, keepdim=True))
     err = d.pow(2).mean(-1).sqrt() / want.std(-1)
     worst = int(err.argmax())
-    assert float(err.max()) <= tol, f"{what}: row {worst} differs by {float(err.max()):.3g} of the logits' spread (limit {tol})"
+    top, usual = tol if isinstance(tol, tuple) else (tol, tol)
+    assert float(err.max()) <= top, f"{what}: row {worst} differs by {float(err.max()):.3g} of the logits' spread (limit {top})"
+    if err.numel() >= 10:
+        nine_in_ten = float(err.kthvalue(int(0.9 * err.numel())).values)
+        assert nine_in_ten <= usual, f"{what}: one row in ten differs by {nine_in_ten:.3g} or more (limit {usual})"
 
 
 def check_trace(folder, ops, prompts, steps, tol, want=None, max_rows=4, block_size=16, num_blocks=None, max_len=512, what=""):
