@@ -44,7 +44,7 @@ def build_engine(cfg_dict, dtype, max_batch, max_len, seed, compile_, chunk=2048
     from socrates_amd.parts import DecoderModel, cache_needs, expected_tensors
     from socrates_amd.weights import random_tensors
 
-    config = config_class_for(cfg_dict["architectures"][0]).from_dict(cfg_dict)
+    config = config_class_for((cfg_dict.get("architectures") or [cfg_dict.get("architecture")])[0]).from_dict(cfg_dict)
     plan = config.plan()
     ops = HipKernels(dtype, "cuda:0")
     weights = random_tensors(expected_tensors(plan), seed, dtype=dtype, device="cuda:0")
@@ -235,6 +235,70 @@ def other_sizes(args, dtype, item):
     return out
 
 
+def mitisun_dict(width, ff, n_layers, wkv_heads, ssm_heads, attn_heads, window=1024):
+    """A Mitisun of ``n_layers`` layers at a real model's layer sizes: time mixing, a state-space mixer
+    and windowed latent attention in turn (every second attention layer reads the cache of the one
+    before it), head sizes of 64 for the recurrent mixers and 128 + 32 for attention over a latent of 96."""
+    ffn = {"kind": "dense", "ff": ff, "limit": 7.0}
+    attention = {"heads": attn_heads, "dim": 128, "rot_dim": 32, "vdim": 128, "kv_rank": 96, "q_rank": width // 4,
+                 "scale": 160 ** -0.5, "rot": {"base": 10000.0, "dims": 32}, "mask": {"size": window}}
+    kinds = [{"type": "wkv", "mixer": {"heads": wkv_heads, "dim": 64, "decay_rank": 64}},
+             {"type": "mamba2", "mixer": {"heads": ssm_heads, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}},
+             {"type": "latent_attention", "mixer": attention}]
+    layers, last_attention = [], None
+    for i in range(n_layers):
+        layer = json.loads(json.dumps(kinds[i % 3]))
+        if layer["type"] == "latent_attention":
+            if last_attention is not None:
+                layer["mixer"]["kv_from"], last_attention = last_attention, None
+            else:
+                last_attention = i
+        layer["mlp"] = dict(ffn)
+        layers.append(layer)
+    return {"architecture": "Mitisun", "vocab": 151936, "width": width, "layers": layers, "norm": {"eps": 1e-6},
+            "residual_mult": 0.5}
+
+
+def mitisun_beside_qwen3(args, dtype, item):
+    """Prefill and decode of Mitisun at a few real layer sizes, each beside Qwen3 of the same width,
+    feed-forward size, vocabulary and number of layers. One JSON line of its own; the default
+    workload's line and contract are untouched."""
+    import torch
+    sizes = [("4b", "qwen3-4b", dict(wkv_heads=40, ssm_heads=80, attn_heads=20)),
+             ("8b", "qwen3-8b", dict(wkv_heads=64, ssm_heads=128, attn_heads=32))]
+    n_layers = args.layers or 12
+    out = {"metric": "prefill and decode of Mitisun beside Qwen3 at equal width, feed-forward, vocabulary and layers",
+           "dtype": args.dtype, "layers": n_layers, "batch": args.batch, "context": args.context,
+           "prefill_tokens": args.prefill_tokens, "data": "synthetic: seeded random weights, uniform random token ids",
+           "sizes": {}}
+    for tag, preset, heads in sizes:
+        q = preset_dict(preset)
+        q["num_hidden_layers"] = n_layers
+        m = mitisun_dict(q["hidden_size"], q["intermediate_size"], n_layers, **heads)
+        point = {}
+        for name, cfg in (("qwen3", q), ("mitisun", m)):
+            config, engine = build_engine(cfg, dtype, args.batch, args.max_len, seed=0, compile_=not args.no_graphs,
+                                          chunk=max(2048, args.prefill_tokens), block_size=args.block_size)
+            V = cfg.get("vocab_size") or cfg["vocab"]
+            if args.dtype == "bf16" and not args.no_tune:
+                engine.tune([args.prefill_tokens, args.batch])
+            tok_s, ms = decode_rate(engine, args.batch, args.context, args.steps, args.warmup, V, seed=1)
+            pre_s = prefill_rate(engine, args.prefill_tokens, V, seed=2)
+            weights = config.param_counts()["read_per_step"] * item
+            cache = (args.batch * args.context * config.kv_bytes_per_token(item) if name == "qwen3"
+                     else config.step_cache_bytes(args.batch, args.context, item))
+            point[name] = {"decode_tok_s": round(tok_s, 1), "decode_ms": round(ms, 4),
+                           "decode_hbm_frac": round((weights + cache) / (ms * 1e-3) / 1e9 / HBM_GBPS, 4),
+                           "prefill_ms": round(pre_s * 1e3, 3), "prefill_tok_s": round(args.prefill_tokens / pre_s, 1),
+                           "prefill_flop_frac": round(config.prefill_flops(args.prefill_tokens) / pre_s / PEAK_FLOPS[args.dtype], 4),
+                           "weights_gb": round(weights / 1e9, 3)}
+            release(engine)
+            torch.cuda.synchronize()
+        out["sizes"][tag] = point
+    print(json.dumps(out))
+    return 0
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -251,6 +315,9 @@ def main(argv=None):
     ap.add_argument("--new-tokens", type=int, default=128, help="--mixed: tokens generated per request")
     ap.add_argument("--decode-rows", type=int, default=64, help="--mixed: requests that decode side by side")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has")
+    ap.add_argument("--mitisun", action="store_true",
+                    help="instead of the default workload: prefill and decode of Mitisun at 4B- and 8B-sized layers "
+                         "(--layers of them, default 12), each beside Qwen3 of the same sizes")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per page of the cache (the reference's 16)")
     ap.add_argument("--no-graphs", action="store_true")
@@ -278,6 +345,8 @@ def main(argv=None):
     import torch
     dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
     item = 2 if args.dtype == "bf16" else 4
+    if args.mitisun:
+        return mitisun_beside_qwen3(args, dtype, item)
     if args.mixed:
         args.preset = args.preset or MIXED_PRESET
         args.max_len = max(args.max_len, 8192)

@@ -178,6 +178,43 @@ class MitisunConfig:
             per_step += 0 if name == "embed" else n
         return {"total": total, "read_per_step": per_step}
 
+    def step_cache_bytes(self, batch: int, context: int, item: int) -> int:
+        """Bytes of cache and state a decode step of ``batch`` requests behind ``context`` tokens reads:
+        the recurrent layers' float32 states, and per attention layer the cached vectors its window sees."""
+        from ..parts import cache_needs
+        from ..parts.registry import PagedLatent, RowState
+        plan = self.plan()
+        needs = cache_needs(plan)
+        total = 0
+        for step in plan.order:
+            need = needs[step.cache]
+            if isinstance(need, RowState):
+                total += 4 * need.shape[0]
+            elif isinstance(need, PagedLatent):
+                window = plan.layers[step.layer].mixer.window
+                total += item * need.width * min(context, window or context)
+        return batch * total
+
+    def prefill_flops(self, tokens: int) -> float:
+        """Multiply-adds times two of one prompt of ``tokens`` tokens from position 0: the matrices
+        (every stored matrix once per token; the head at one position), attention scores and sums over
+        each window, and the two recurrences (per token and head, state size times four)."""
+        from ..parts import expected_tensors
+        plan = self.plan()
+        matrices = sum(decl.shape[0] * decl.shape[1] for name, decl in expected_tensors(plan).items()
+                       if decl.kind == "matrix" and len(decl.shape) == 2 and name not in ("embed", "head") and -1 not in decl.shape)
+        flops = 2.0 * tokens * matrices + 2.0 * self.vocab * self.width
+        for block in plan.layers:
+            m = block.mixer
+            if isinstance(m, LatentAttentionSpec):
+                seen = sum(min(p + 1, m.window or p + 1) for p in range(tokens))
+                flops += 2.0 * seen * m.n_heads * (m.cache_width + m.kv_rank)
+            elif isinstance(m, WkvSpec):
+                flops += 4.0 * tokens * m.n_heads * m.head_dim * m.head_dim
+            elif isinstance(m, Mamba2Spec):
+                flops += 4.0 * tokens * m.n_heads * m.state * m.head_dim
+        return flops
+
 
 def _freeze(x):
     if isinstance(x, dict):

@@ -161,88 +161,269 @@ SOC_EXPORT int soc_wkv_decay(const float* t, const void* w2, const float* w0, fl
     return soc_last_error();
 }
 
-// ---- recurrence with a decay per key channel -------------------------------------------------------
-// Per (head, sequence): thread j owns column j of the state S [D keys, D values] in registers.
-// o_t[j] = sum_i r_t[i] (S[i, j] + u[i] k_t[i] v_t[j]); S[i, j] <- w_t[i] S[i, j] + k_t[i] v_t[j].
-// Then o over its root mean square over the head, times gain, times silu(g).
-template <typename T, int DK>
-__global__ void __launch_bounds__(256)
-wkv_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ decay,
-           const T* __restrict__ g, const float* __restrict__ bonus, const float* __restrict__ gain, float eps,
-           int H, int D, float* __restrict__ state, size_t stride, int offset, const int* __restrict__ seq_qstart,
-           const int* __restrict__ seq_rows, T* __restrict__ out) {
-    __shared__ float sr[DK], sk[DK], sw[DK], su[DK], scratch[16];
-    const int head = blockIdx.x, seq = blockIdx.y, j = threadIdx.x;
-    const int lo = seq_qstart[seq], hi = seq_qstart[seq + 1];
-    if (lo >= hi) return;
-    const bool live = j < D;
-    float* S = state + (size_t)seq_rows[seq] * stride + offset + (size_t)head * D * D;
-    float s[DK];
-#pragma unroll
-    for (int i = 0; i < DK; ++i) s[i] = (live && i < D) ? S[(size_t)i * D + j] : 0.f;
-    if (j < DK) su[j] = live ? bonus[head * D + j] : 0.f;
-    const size_t C = (size_t)H * D;
-    for (int n = lo; n < hi; ++n) {
-        const size_t at = (size_t)n * C + (size_t)head * D + j;
-        __syncthreads();
-        if (j < DK) {
-            sr[j] = live ? to_float(r[at]) : 0.f;
-            sk[j] = live ? to_float(k[at]) : 0.f;
-            sw[j] = live ? decay[at] : 0.f;
-        }
-        __syncthreads();
-        const float vj = live ? to_float(v[at]) : 0.f;
-        float o = 0.f;
-#pragma unroll
-        for (int i = 0; i < DK; ++i) {
-            const float kv = sk[i] * vj;
-            o = fmaf(sr[i], fmaf(su[i], kv, s[i]), o);
-            s[i] = fmaf(sw[i], s[i], kv);
-        }
-        const float ss = block_sum(live ? o * o : 0.f, scratch);
-        if (live) {
-            const float gate = to_float(g[at]);
-            out[at] = from_float<T>(o / sqrtf(ss / (float)D + eps) * gain[head * D + j] * gate * soc_sigmoid(gate));
-        }
-    }
-    if (live) {
-#pragma unroll
-        for (int i = 0; i < DK; ++i)
-            if (i < D) S[(size_t)i * D + j] = s[i];
-    }
-}
+// ---- the two recurrences with a matrix state per head ---------------------------------------------------
+// A workgroup of 256 threads owns CW columns of one head's state S [keys, columns] for one sequence, in
+// registers: thread (part, column) holds keys part * KPT .. (part + 1) * KPT - 1 of its column (PARTS * CW =
+// 256; consecutive lanes are consecutive columns). Columns never meet in the recurrence, so a head is
+// spread over as many workgroups as fill the GPU (CW = 16 when sequences and heads alone give too few,
+// else 64). Tokens go in batches: what all threads need of a batch (per key: r, k, decay; or B,
+// C) is staged through LDS; the next batch's global loads are issued before the current batch is computed
+// and land in LDS after it; the partial sums of a column's PARTS threads meet in LDS once per batch.
+// (tokens per batch: 16 for states of up to 64 keys, else 8: what LDS holds twice over)
+constexpr int rec_batch(int keys) { return keys <= 64 ? 16 : 8; }
 
-template <typename T, int DK>
-static void launch_wkv(const void* r, const void* k, const void* v, const float* decay, const void* g, const float* bonus,
-                       const float* gain, float eps, int H, int D, float* state, long long stride, int offset,
-                       const int* seq_qstart, const int* seq_rows, void* out, int n_seqs, hipStream_t stream) {
-    const int threads = (max(D, DK) + 63) / 64 * 64;
-    hipLaunchKernelGGL((wkv_kernel<T, DK>), dim3(H, n_seqs), dim3(threads), 0, stream, (const T*)r, (const T*)k,
-                       (const T*)v, decay, (const T*)g, bonus, gain, eps, H, D, state, (size_t)stride, offset, seq_qstart,
-                       seq_rows, (T*)out);
-}
+// A barrier for threads that meet in LDS only: a wave waits for its own LDS accesses, not for its global
+// loads and stores in flight (__syncthreads waits for those too, which would drain the next batch's
+// loads, issued on purpose before the current batch is computed, at every barrier).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 #define SOC_BY_STATE_SIZE(D, CALL)                                         \
     switch (((D) + 15) / 16) {                                              \
         case 1: CALL(16); break;   case 2: CALL(32); break;                 \
         case 3: CALL(48); break;   case 4: CALL(64); break;                 \
-        case 5: CALL(80); break;   case 6: CALL(96); break;                 \
-        case 7: CALL(112); break;  case 8: CALL(128); break;                \
-        case 9: case 10: CALL(160); break;                                  \
-        case 11: case 12: CALL(192); break;                                 \
-        case 13: case 14: CALL(224); break;                                 \
-        case 15: case 16: CALL(256); break;                                 \
+        case 5: case 6: CALL(96); break;                                    \
+        case 7: case 8: CALL(128); break;                                   \
+        case 9: case 10: case 11: case 12: CALL(192); break;                \
+        case 13: case 14: case 15: case 16: CALL(256); break;               \
         default: return (int)hipErrorInvalidValue;                          \
     }
 
-SOC_EXPORT int soc_wkv(const void* r, const void* k, const void* v, const float* decay, const void* g, const float* bonus,
-                       const float* gain, float eps, int H, int D, float* state, long long stride, int offset,
-                       const int* seq_qstart, const int* seq_rows, void* out, int n_seqs, int dtype, hipStream_t stream) {
+// Decay per key channel: o_t[j] = sum_i r_t[i] (S[i, j] + u[i] k_t[i] v_t[j]); S[i, j] <- w_t[i] S[i, j] +
+// k_t[i] v_t[j]. o goes out in float32; its norm over the head is another kernel's.
+template <typename T, int DK, int CW>
+__global__ void __launch_bounds__(256)
+wkv_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* __restrict__ v, const float* __restrict__ decay,
+           const float* __restrict__ bonus, int H, int D, float* __restrict__ state, size_t stride, int offset,
+           const int* __restrict__ seq_qstart, const int* __restrict__ seq_rows, float* __restrict__ out) {
+    constexpr int REC_TB = rec_batch(DK), PARTS = 256 / CW, KPT = DK / PARTS, STAGE = (REC_TB * DK + 255) / 256;
+    __shared__ float sr[2][REC_TB][DK], sk[2][REC_TB][DK], sw[2][REC_TB][DK];
+    __shared__ float red[REC_TB][PARTS][CW], su[DK];
+    const int blocks = (D + CW - 1) / CW;
+    const int head = blockIdx.x / blocks, seq = blockIdx.y, tid = threadIdx.x;
+    const int lo = seq_qstart[seq], hi = seq_qstart[seq + 1];
+    if (lo >= hi) return;
+    const int col0 = (blockIdx.x % blocks) * CW;
+    const int col = col0 + tid % CW, part = tid / CW, i0 = part * KPT;
+    const bool live = col < D;
+    float* S = state + (size_t)seq_rows[seq] * stride + offset + (size_t)head * D * D;
+    const size_t C = (size_t)H * D, hoff = (size_t)head * D;
+    float s[KPT];
+#pragma unroll
+    for (int ii = 0; ii < KPT; ++ii) s[ii] = (live && i0 + ii < D) ? S[(size_t)(i0 + ii) * D + col] : 0.f;
+    for (int i = tid; i < DK; i += 256) su[i] = i < D ? bonus[head * D + i] : 0.f;
+
+    float fr[STAGE], fk[STAGE], fw[STAGE], fv[REC_TB];
+    auto fetch = [&](int n0) {
+#pragma unroll
+        for (int q = 0; q < STAGE; ++q) {
+            const int e = tid + q * 256, t = e / DK, i = e % DK;
+            const bool in = t < REC_TB && n0 + t < hi && i < D;
+            const size_t at = (size_t)(n0 + t) * C + hoff + i;
+            fr[q] = in ? to_float(r[at]) : 0.f;
+            fk[q] = in ? to_float(k[at]) : 0.f;
+            fw[q] = in ? decay[at] : 0.f;
+        }
+#pragma unroll
+        for (int t = 0; t < REC_TB; ++t)
+            fv[t] = (live && n0 + t < hi) ? to_float(v[(size_t)(n0 + t) * C + hoff + col]) : 0.f;
+    };
+    auto land = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < STAGE; ++q) {
+            const int e = tid + q * 256, t = e / DK, i = e % DK;
+            if (t < REC_TB) { sr[buf][t][i] = fr[q]; sk[buf][t][i] = fk[q]; sw[buf][t][i] = fw[q]; }
+        }
+    };
+    fetch(lo);
+    land(0);
+    lds_barrier();
+    int buf = 0;
+    for (int n0 = lo; n0 < hi; n0 += REC_TB, buf ^= 1) {
+        const int nb = min(REC_TB, hi - n0);
+        const bool more = n0 + REC_TB < hi;
+        float vj[REC_TB];
+#pragma unroll
+        for (int t = 0; t < REC_TB; ++t) vj[t] = fv[t];
+        if (more) fetch(n0 + REC_TB);
+#pragma unroll
+        for (int t = 0; t < REC_TB; ++t) {
+            if (t < nb) {
+                float acc = 0.f;
+#pragma unroll
+                for (int ii = 0; ii < KPT; ++ii) {
+                    const float kv = sk[buf][t][i0 + ii] * vj[t];
+                    acc = fmaf(sr[buf][t][i0 + ii], fmaf(su[i0 + ii], kv, s[ii]), acc);
+                    s[ii] = fmaf(sw[buf][t][i0 + ii], s[ii], kv);
+                }
+                red[t][part][tid % CW] = acc;
+            }
+        }
+        lds_barrier();
+        for (int f = tid; f < REC_TB * CW; f += 256) {
+            const int t = f / CW, cl = f % CW;
+            if (t < nb && col0 + cl < D) {
+                float o = 0.f;
+#pragma unroll
+                for (int pp = 0; pp < PARTS; ++pp) o += red[t][pp][cl];
+                out[(size_t)(n0 + t) * C + hoff + col0 + cl] = o;
+            }
+        }
+        if (more) land(buf ^ 1);
+        lds_barrier();
+    }
+    if (live) {
+#pragma unroll
+        for (int ii = 0; ii < KPT; ++ii)
+            if (i0 + ii < D) S[(size_t)(i0 + ii) * D + col] = s[ii];
+    }
+}
+
+template <typename T, int DK>
+static void launch_wkv(const void* r, const void* k, const void* v, const float* decay, const float* bonus, int H, int D,
+                       float* state, long long stride, int offset, const int* seq_qstart, const int* seq_rows, float* out,
+                       int n_seqs, int cw, hipStream_t stream) {
+#define SOC_WKV_LAUNCH(CW)                                                                                                  \
+    hipLaunchKernelGGL((wkv_kernel<T, DK, CW>), dim3(H * ((D + CW - 1) / CW), n_seqs), dim3(256), 0, stream, (const T*)r, \
+                       (const T*)k, (const T*)v, decay, bonus, H, D, state, (size_t)stride, offset, seq_qstart, seq_rows, out)
+    if (cw == 16) SOC_WKV_LAUNCH(16); else SOC_WKV_LAUNCH(64);
+}
+
+// Columns per workgroup: 64, or 16 where heads and sequences alone leave most compute units idle.
+// (A step with a prompt portion in it is as long as that portion's walk, whatever else is in the step.)
+static int columns_per_workgroup(int H, int cols, int n_seqs, int max_q_len) {
+    if (max_q_len > 64) return 16;
+    return (long long)H * ((cols + 63) / 64) * n_seqs >= 192 ? 64 : 16;
+}
+
+SOC_EXPORT int soc_wkv(const void* r, const void* k, const void* v, const float* decay, const float* bonus, int H, int D,
+                       float* state, long long stride, int offset, const int* seq_qstart, const int* seq_rows, float* out,
+                       int n_seqs, int max_q_len, int dtype, hipStream_t stream) {
     if (n_seqs <= 0 || H <= 0) return 0;
-    if (D < 1 || D > 256) return (int)hipErrorInvalidValue;
-#define SOC_WKV_F32(DK) launch_wkv<float, DK>(r, k, v, decay, g, bonus, gain, eps, H, D, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, stream)
-#define SOC_WKV_BF16(DK) launch_wkv<bf16, DK>(r, k, v, decay, g, bonus, gain, eps, H, D, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, stream)
+    if (D < 1 || D > 256 || n_seqs > 65535) return (int)hipErrorInvalidValue;
+    const int cw = columns_per_workgroup(H, D, n_seqs, max_q_len);
+#define SOC_WKV_F32(DK) launch_wkv<float, DK>(r, k, v, decay, bonus, H, D, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, cw, stream)
+#define SOC_WKV_BF16(DK) launch_wkv<bf16, DK>(r, k, v, decay, bonus, H, D, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, cw, stream)
     if (dtype == 0) { SOC_BY_STATE_SIZE(D, SOC_WKV_F32) } else { SOC_BY_STATE_SIZE(D, SOC_WKV_BF16) }
+    return soc_last_error();
+}
+
+// Scalar decay per head: xbc [N, x (H P) | B (G Ns) | C (G Ns)]; dt = softplus(dt_raw + bias);
+// S[i, p] <- exp(-exp(a_log) dt) S[i, p] + dt B[i] x[p]; y[p] = sum_i C[i] S[i, p] + skip x[p], float32.
+template <typename T, int NK, int CW>
+__global__ void __launch_bounds__(256)
+ssd_kernel(const T* __restrict__ xbc, const float* __restrict__ dt_raw, const float* __restrict__ dt_bias,
+           const float* __restrict__ a_log, const float* __restrict__ skip, int H, int P, int Ns, int G,
+           float* __restrict__ state, size_t stride, int offset, const int* __restrict__ seq_qstart,
+           const int* __restrict__ seq_rows, float* __restrict__ out) {
+    constexpr int REC_TB = rec_batch(NK), PARTS = 256 / CW, KPT = NK / PARTS, STAGE = (REC_TB * NK + 255) / 256;
+    __shared__ float sb[2][REC_TB][NK], sc[2][REC_TB][NK], skeep[2][REC_TB];
+    __shared__ float red[REC_TB][PARTS][CW];
+    const int blocks = (P + CW - 1) / CW;
+    const int head = blockIdx.x / blocks, seq = blockIdx.y, tid = threadIdx.x;
+    const int lo = seq_qstart[seq], hi = seq_qstart[seq + 1];
+    if (lo >= hi) return;
+    const int col0 = (blockIdx.x % blocks) * CW;
+    const int col = col0 + tid % CW, part = tid / CW, i0 = part * KPT;
+    const bool live = col < P;
+    const int group = head / (H / G);
+    const int inner = H * P, ld = inner + 2 * G * Ns;
+    const int boff = inner + group * Ns, coff = inner + G * Ns + group * Ns;
+    float* S = state + (size_t)seq_rows[seq] * stride + offset + (size_t)head * Ns * P;
+    float s[KPT];
+#pragma unroll
+    for (int ii = 0; ii < KPT; ++ii) s[ii] = (live && i0 + ii < Ns) ? S[(size_t)(i0 + ii) * P + col] : 0.f;
+    const float rate = expf(a_log[head]), through = skip[head], shift = dt_bias[head];
+    auto step_size = [&](int n) {
+        const float z = dt_raw[(size_t)n * H + head] + shift;
+        return z > 20.f ? z : log1pf(expf(z));
+    };
+
+    float fb[STAGE], fc[STAGE], fx[REC_TB], fkeep = 0.f;
+    auto fetch = [&](int n0) {
+#pragma unroll
+        for (int t = 0; t < REC_TB; ++t)
+            fx[t] = (live && n0 + t < hi) ? to_float(xbc[(size_t)(n0 + t) * ld + head * P + col]) : 0.f;
+#pragma unroll
+        for (int q = 0; q < STAGE; ++q) {
+            const int e = tid + q * 256, t = e / NK, i = e % NK;
+            const bool in = t < REC_TB && n0 + t < hi && i < Ns;
+            const T* row = xbc + (size_t)(n0 + t) * ld;
+            fb[q] = in ? step_size(n0 + t) * to_float(row[boff + i]) : 0.f;
+            fc[q] = in ? to_float(row[coff + i]) : 0.f;
+        }
+        if (tid < REC_TB) fkeep = n0 + tid < hi ? expf(-rate * step_size(n0 + tid)) : 1.f;
+    };
+    auto land = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < STAGE; ++q) {
+            const int e = tid + q * 256, t = e / NK, i = e % NK;
+            if (t < REC_TB) { sb[buf][t][i] = fb[q]; sc[buf][t][i] = fc[q]; }
+        }
+        if (tid < REC_TB) skeep[buf][tid] = fkeep;
+    };
+    fetch(lo);
+    land(0);
+    lds_barrier();
+    int buf = 0;
+    for (int n0 = lo; n0 < hi; n0 += REC_TB, buf ^= 1) {
+        const int nb = min(REC_TB, hi - n0);
+        const bool more = n0 + REC_TB < hi;
+        float xj[REC_TB];
+#pragma unroll
+        for (int t = 0; t < REC_TB; ++t) xj[t] = fx[t];
+        if (more) fetch(n0 + REC_TB);
+#pragma unroll
+        for (int t = 0; t < REC_TB; ++t) {
+            if (t < nb) {
+                const float keep = skeep[buf][t];
+                float acc = part == 0 ? through * xj[t] : 0.f;
+#pragma unroll
+                for (int ii = 0; ii < KPT; ++ii) {
+                    s[ii] = fmaf(keep, s[ii], sb[buf][t][i0 + ii] * xj[t]);
+                    acc = fmaf(sc[buf][t][i0 + ii], s[ii], acc);
+                }
+                red[t][part][tid % CW] = acc;
+            }
+        }
+        lds_barrier();
+        for (int f = tid; f < REC_TB * CW; f += 256) {
+            const int t = f / CW, cl = f % CW;
+            if (t < nb && col0 + cl < P) {
+                float y = 0.f;
+#pragma unroll
+                for (int pp = 0; pp < PARTS; ++pp) y += red[t][pp][cl];
+                out[(size_t)(n0 + t) * inner + head * P + col0 + cl] = y;
+            }
+        }
+        if (more) land(buf ^ 1);
+        lds_barrier();
+    }
+    if (live) {
+#pragma unroll
+        for (int ii = 0; ii < KPT; ++ii)
+            if (i0 + ii < Ns) S[(size_t)(i0 + ii) * P + col] = s[ii];
+    }
+}
+
+template <typename T, int NK>
+static void launch_ssd(const void* xbc, const float* dt_raw, const float* dt_bias, const float* a_log, const float* skip,
+                       int H, int P, int Ns, int G, float* state, long long stride, int offset, const int* seq_qstart,
+                       const int* seq_rows, float* out, int n_seqs, int cw, hipStream_t stream) {
+#define SOC_SSD_LAUNCH(CW)                                                                                                   \
+    hipLaunchKernelGGL((ssd_kernel<T, NK, CW>), dim3(H * ((P + CW - 1) / CW), n_seqs), dim3(256), 0, stream, (const T*)xbc, \
+                       dt_raw, dt_bias, a_log, skip, H, P, Ns, G, state, (size_t)stride, offset, seq_qstart, seq_rows, out)
+    if (cw == 16) SOC_SSD_LAUNCH(16); else SOC_SSD_LAUNCH(64);
+}
+
+SOC_EXPORT int soc_ssd(const void* xbc, const float* dt_raw, const float* dt_bias, const float* a_log, const float* skip,
+                       int H, int P, int Ns, int G, float* state, long long stride, int offset, const int* seq_qstart,
+                       const int* seq_rows, float* out, int n_seqs, int max_q_len, int dtype, hipStream_t stream) {
+    if (n_seqs <= 0 || H <= 0) return 0;
+    if (Ns < 1 || Ns > 256 || P < 1 || G < 1 || H % G || n_seqs > 65535) return (int)hipErrorInvalidValue;
+    const int cw = columns_per_workgroup(H, P, n_seqs, max_q_len);
+#define SOC_SSD_F32(NK) launch_ssd<float, NK>(xbc, dt_raw, dt_bias, a_log, skip, H, P, Ns, G, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, cw, stream)
+#define SOC_SSD_BF16(NK) launch_ssd<bf16, NK>(xbc, dt_raw, dt_bias, a_log, skip, H, P, Ns, G, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, cw, stream)
+    if (dtype == 0) { SOC_BY_STATE_SIZE(Ns, SOC_SSD_F32) } else { SOC_BY_STATE_SIZE(Ns, SOC_SSD_BF16) }
     return soc_last_error();
 }
 
@@ -302,93 +483,26 @@ SOC_EXPORT int soc_causal_conv_silu(const void* x, int ldx, int col, int C, cons
     return soc_last_error();
 }
 
-// ---- recurrence with a scalar decay per head -------------------------------------------------------------
-// xbc [N, x (H P) | B (G Ns) | C (G Ns)]; dt = softplus(dt_raw + bias). Per (head, sequence): thread p
-// owns column p of S [Ns, P]: S[i, p] <- exp(-exp(a_log) dt) S[i, p] + dt B[i] x[p];
-// y[p] = sum_i C[i] S[i, p] + skip x[p], float32.
-template <typename T, int NK>
-__global__ void __launch_bounds__(256)
-ssd_kernel(const T* __restrict__ xbc, const float* __restrict__ dt_raw, const float* __restrict__ dt_bias,
-           const float* __restrict__ a_log, const float* __restrict__ skip, int H, int P, int Ns, int G,
-           float* __restrict__ state, size_t stride, int offset, const int* __restrict__ seq_qstart,
-           const int* __restrict__ seq_rows, float* __restrict__ out) {
-    __shared__ float sb[NK], sc[NK];
-    const int head = blockIdx.x, seq = blockIdx.y, p = threadIdx.x;
-    const int lo = seq_qstart[seq], hi = seq_qstart[seq + 1];
-    if (lo >= hi) return;
-    const bool live = p < P;
-    const int group = head / (H / G);
-    const int inner = H * P, ld = inner + 2 * G * Ns;
-    float* S = state + (size_t)seq_rows[seq] * stride + offset + (size_t)head * Ns * P;
-    float s[NK];
-#pragma unroll
-    for (int i = 0; i < NK; ++i) s[i] = (live && i < Ns) ? S[(size_t)i * P + p] : 0.f;
-    const float rate = expf(a_log[head]), through = skip[head], shift = dt_bias[head];
-    for (int n = lo; n < hi; ++n) {
-        const float z = dt_raw[(size_t)n * H + head] + shift;
-        const float dt = z > 20.f ? z : log1pf(expf(z));
-        const float keep = expf(-rate * dt);
-        const T* row = xbc + (size_t)n * ld;
-        __syncthreads();
-        if (p < NK) {
-            const bool in = p < Ns;
-            sb[p] = in ? dt * to_float(row[inner + group * Ns + p]) : 0.f;
-            sc[p] = in ? to_float(row[inner + G * Ns + group * Ns + p]) : 0.f;
-        }
-        __syncthreads();
-        const float xp = live ? to_float(row[head * P + p]) : 0.f;
-        float y = through * xp;
-#pragma unroll
-        for (int i = 0; i < NK; ++i) {
-            s[i] = fmaf(keep, s[i], sb[i] * xp);
-            y = fmaf(sc[i], s[i], y);
-        }
-        if (live) out[(size_t)n * inner + head * P + p] = y;
-    }
-    if (live) {
-#pragma unroll
-        for (int i = 0; i < NK; ++i)
-            if (i < Ns) S[(size_t)i * P + p] = s[i];
-    }
-}
-
-template <typename T, int NK>
-static void launch_ssd(const void* xbc, const float* dt_raw, const float* dt_bias, const float* a_log, const float* skip,
-                       int H, int P, int Ns, int G, float* state, long long stride, int offset, const int* seq_qstart,
-                       const int* seq_rows, float* out, int n_seqs, hipStream_t stream) {
-    const int threads = (max(P, NK) + 63) / 64 * 64;
-    hipLaunchKernelGGL((ssd_kernel<T, NK>), dim3(H, n_seqs), dim3(threads), 0, stream, (const T*)xbc, dt_raw, dt_bias, a_log,
-                       skip, H, P, Ns, G, state, (size_t)stride, offset, seq_qstart, seq_rows, out);
-}
-
-SOC_EXPORT int soc_ssd(const void* xbc, const float* dt_raw, const float* dt_bias, const float* a_log, const float* skip,
-                       int H, int P, int Ns, int G, float* state, long long stride, int offset, const int* seq_qstart,
-                       const int* seq_rows, float* out, int n_seqs, int dtype, hipStream_t stream) {
-    if (n_seqs <= 0 || H <= 0) return 0;
-    if (Ns < 1 || Ns > 256 || P < 1 || P > 256 || G < 1 || H % G) return (int)hipErrorInvalidValue;
-#define SOC_SSD_F32(NK) launch_ssd<float, NK>(xbc, dt_raw, dt_bias, a_log, skip, H, P, Ns, G, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, stream)
-#define SOC_SSD_BF16(NK) launch_ssd<bf16, NK>(xbc, dt_raw, dt_bias, a_log, skip, H, P, Ns, G, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, stream)
-    if (dtype == 0) { SOC_BY_STATE_SIZE(Ns, SOC_SSD_F32) } else { SOC_BY_STATE_SIZE(Ns, SOC_SSD_BF16) }
-    return soc_last_error();
-}
-
-// ---- y * silu(z), then RMS norm in equal parts, times gain ------------------------------------------------
-// y float32 [N, inner]; z the first `inner` columns of rows of ldz elements. One workgroup per (part, token).
-template <typename T>
+// ---- RMS norm in equal parts with a gate silu(z), in front of the norm or behind it ------------------------
+// y float32 [N, inner]; z the first `inner` columns of rows of ldz elements. Gate first: norm(y silu(z)) gain;
+// gate last: norm(y) gain silu(z). One wave per (part, token), WAVES of them in a workgroup.
+template <typename T, bool GATE_FIRST>
 __global__ void __launch_bounds__(256)
 gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, int ldz, const float* __restrict__ gain,
-                        int inner, int part, float eps, T* __restrict__ out) {
-    __shared__ float scratch[16];
-    const int n = blockIdx.y, c0 = blockIdx.x * part;
+                        int inner, int part, int n_items, float eps, T* __restrict__ out) {
+    const int item = blockIdx.x * (blockDim.x / SOC_WAVE) + threadIdx.x / SOC_WAVE, lane = threadIdx.x % SOC_WAVE;
+    if (item >= n_items) return;
+    const int parts = inner / part;
+    const int n = item / parts, c0 = (item % parts) * part;
     float ss = 0.f;
-    for (int c = c0 + threadIdx.x; c < c0 + part; c += blockDim.x) {
-        const float zz = to_float(z[(size_t)n * ldz + c]);
-        const float v = y[(size_t)n * inner + c] * zz * soc_sigmoid(zz);
+    for (int c = c0 + lane; c < c0 + part; c += SOC_WAVE) {
+        float v = y[(size_t)n * inner + c];
+        if (GATE_FIRST) { const float zz = to_float(z[(size_t)n * ldz + c]); v *= zz * soc_sigmoid(zz); }
         ss += v * v;
     }
-    ss = block_sum(ss, scratch);
+    ss = wave_sum(ss);
     const float inv = 1.f / sqrtf(ss / (float)part + eps);
-    for (int c = c0 + threadIdx.x; c < c0 + part; c += blockDim.x) {
+    for (int c = c0 + lane; c < c0 + part; c += SOC_WAVE) {
         const float zz = to_float(z[(size_t)n * ldz + c]);
         const float v = y[(size_t)n * inner + c] * zz * soc_sigmoid(zz);
         out[(size_t)n * inner + c] = from_float<T>(v * inv * gain[c]);
@@ -396,16 +510,16 @@ gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, in
 }
 
 SOC_EXPORT int soc_gated_group_norm(const float* y, const void* z, int ldz, const float* gain, int N, int inner, int parts,
-                                    float eps, void* out, int dtype, hipStream_t stream) {
+                                    float eps, int gate_first, void* out, int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
-    if (parts < 1 || inner % parts) return (int)hipErrorInvalidValue;
-    const dim3 grid(parts, N);
-    if (dtype == 0)
-        hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, dim3(256), 0, stream, y, (const float*)z, ldz, gain, inner,
-                           inner / parts, eps, (float*)out);
-    else
-        hipLaunchKernelGGL(gated_group_norm_kernel<bf16>, grid, dim3(256), 0, stream, y, (const bf16*)z, ldz, gain, inner,
-                           inner / parts, eps, (bf16*)out);
+    if (parts < 1 || inner % parts || (long long)N * parts > 0x7fffffffLL) return (int)hipErrorInvalidValue;
+    const int items = N * parts;
+    const dim3 grid((items + 3) / 4);
+#define SOC_GGN(T, FIRST)                                                                                             \
+    hipLaunchKernelGGL((gated_group_norm_kernel<T, FIRST>), grid, dim3(256), 0, stream, y, (const T*)z, ldz, gain, inner, \
+                       inner / parts, items, eps, (T*)out)
+    if (dtype == 0) { if (gate_first) SOC_GGN(float, true); else SOC_GGN(float, false); }
+    else { if (gate_first) SOC_GGN(bf16, true); else SOC_GGN(bf16, false); }
     return soc_last_error();
 }
 

@@ -105,12 +105,12 @@ class Mixers:
         self._want(bonus, "bonus", torch.float32, (H, D))
         self._want(gain, "gain", torch.float32, (C,))
         stride = self._state(state, offset, H * D * D, ctx)
-        out = torch.empty((N, C), dtype=self.dtype, device=self.device)
-        _check(self._mixers().soc_wkv(_ptr(r), _ptr(k), _ptr(v), _ptr(decay), _ptr(g), _ptr(bonus), _ptr(gain), c_float(eps),
-                                      c_int(H), c_int(D), _ptr(state), stride, c_int(offset), _ptr(ctx.seq_qstart),
-                                      _ptr(ctx.seq_rows), _ptr(out), c_int(ctx.n_seqs), c_int(self.code), self._stream()),
-               "wkv")
-        return out
+        raw = torch.empty((N, C), dtype=torch.float32, device=self.device)
+        _check(self._mixers().soc_wkv(_ptr(r), _ptr(k), _ptr(v), _ptr(decay), _ptr(bonus), c_int(H), c_int(D), _ptr(state),
+                                      stride, c_int(offset), _ptr(ctx.seq_qstart), _ptr(ctx.seq_rows), _ptr(raw),
+                                      c_int(ctx.n_seqs), c_int(ctx.max_q_len), c_int(self.code), self._stream()), "wkv")
+        # (a head's columns are spread over workgroups: its norm is a kernel of its own)
+        return self.gated_group_norm(raw, g, gain, H, eps, gate_first=False)
 
     def causal_conv_silu(self, x, col, C, weight, bias, state, offset, ctx):
         """silu of a causal convolution per channel over columns col .. col + C of ``x``; the row's
@@ -139,17 +139,18 @@ class Mixers:
         self._want(dt, "step sizes", torch.float32, (N, H))
         for t, name in ((dt_bias, "dt bias"), (a_log, "A_log"), (skip, "D")):
             self._want(t, name, torch.float32, (H,))
-        if H % G or not 1 <= Ns <= 256 or not 1 <= P <= 256:
+        if H % G or not 1 <= Ns <= 256 or P < 1:
             raise KernelError(f"ssd: {H} heads in {G} groups, state {Ns}, head size {P}")
         stride = self._state(state, offset, H * Ns * P, ctx)
         out = torch.empty((N, H * P), dtype=torch.float32, device=self.device)
         _check(self._mixers().soc_ssd(_ptr(xbc), _ptr(dt), _ptr(dt_bias), _ptr(a_log), _ptr(skip), c_int(H), c_int(P), c_int(Ns),
                                       c_int(G), _ptr(state), stride, c_int(offset), _ptr(ctx.seq_qstart), _ptr(ctx.seq_rows),
-                                      _ptr(out), c_int(ctx.n_seqs), c_int(self.code), self._stream()), "ssd")
+                                      _ptr(out), c_int(ctx.n_seqs), c_int(ctx.max_q_len), c_int(self.code), self._stream()), "ssd")
         return out
 
-    def gated_group_norm(self, y, z, gain, groups, eps):
-        """y (float32 [N, inner]) * silu(z[:, :inner]), RMS-normed in ``groups`` equal parts, times gain."""
+    def gated_group_norm(self, y, z, gain, groups, eps, gate_first=True):
+        """y (float32 [N, inner]) * silu(z[:, :inner]), RMS-normed in ``groups`` equal parts, times gain;
+        ``gate_first`` False: y normed, times gain, and only then times silu(z)."""
         N, inner = y.shape
         self._want(y, "y", torch.float32)
         self._want(z, "z", self.dtype)
@@ -158,7 +159,8 @@ class Mixers:
             raise KernelError(f"gated norm: z {tuple(z.shape)} against y {tuple(y.shape)} in {groups} parts")
         out = torch.empty((N, inner), dtype=self.dtype, device=self.device)
         _check(self._mixers().soc_gated_group_norm(_ptr(y), _ptr(z), c_int(z.shape[1]), _ptr(gain), c_int(N), c_int(inner),
-                                                   c_int(groups), c_float(eps), _ptr(out), c_int(self.code), self._stream()),
+                                                   c_int(groups), c_float(eps), c_int(1 if gate_first else 0), _ptr(out),
+                                                   c_int(self.code), self._stream()),
                "gated_group_norm")
         return out
 
@@ -196,6 +198,12 @@ class Mixers:
         self._want(out, "out", self.dtype)
         if out.dim() != 3 or out.shape[:2] != (N, H) or out.shape[2] < n_out:
             raise KernelError(f"per-head product: out {tuple(out.shape)}")
+        if (self.dtype == torch.bfloat16 and N > 16 and self.library_gemm and K % 8 == 0 and n_out % 8 == 0
+                and not torch.cuda.is_current_stream_capturing()):
+            # more than 16 rows in bfloat16: the library's batched product, as for every other
+            # product of that size (float32 sums inside); its [H, N, n_out] result is laid back by head
+            out[:, :, :n_out].copy_(torch.bmm(x.transpose(0, 1)[:, :, :K], w.transpose(1, 2)).transpose(0, 1))
+            return out
         _check(self._mixers().soc_head_linear(_ptr(x), c_int(ldx), _ptr(w), _ptr(out), c_int(out.shape[2]), c_int(N), c_int(H),
                                               c_int(n_out), c_int(K), c_int(self.code), self._stream()), "head_linear")
         return out
