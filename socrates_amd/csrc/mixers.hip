@@ -133,7 +133,8 @@ SOC_EXPORT int soc_token_shift(const void* h, const float* mu, int n_streams, fl
 }
 
 // ---- decay = exp(-exp(tanh(t) W2^T + w0)) --------------------------------------------------------
-// t [N, rank] float32; W2 [C, rank]; one workgroup per token keeps tanh(t) in LDS.
+// t [N, rank] float32; W2 transposed, [rank, C] (consecutive threads read consecutive elements); one
+// workgroup per token keeps tanh(t) in LDS.
 template <typename T>
 __global__ void __launch_bounds__(256)
 wkv_decay_kernel(const float* __restrict__ t, const T* __restrict__ w2, const float* __restrict__ w0,
@@ -144,8 +145,7 @@ wkv_decay_kernel(const float* __restrict__ t, const T* __restrict__ w2, const fl
     __syncthreads();
     for (int c = threadIdx.x; c < C; c += blockDim.x) {
         float z = 0.f;
-        const T* row = w2 + (size_t)c * rank;
-        for (int j = 0; j < rank; ++j) z = fmaf(th[j], to_float(row[j]), z);
+        for (int j = 0; j < rank; ++j) z = fmaf(th[j], to_float(w2[(size_t)j * C + c]), z);
         out[(size_t)n * C + c] = expf(-expf(z + w0[c]));
     }
 }

@@ -77,13 +77,14 @@ class Mixers:
                "token_shift")
         return out
 
-    def wkv_decay(self, t, w2, w0):
-        """float32 [N, C]: exp(-exp(tanh(t) w2^T + w0)); t float32 [N, rank]."""
+    def wkv_decay(self, t, w2_t, w0):
+        """float32 [N, C]: exp(-exp(tanh(t) w2 + w0)); t float32 [N, rank], ``w2_t`` [rank, C] (the stored
+        matrix transposed, so that consecutive outputs read consecutive elements)."""
         N, rank = t.shape
         self._want(t, "decay latent", torch.float32)
-        self._want(w2, "decay matrix")
-        C = w2.shape[0]
-        if w2.shape != (C, rank) or w2.dtype not in _DTYPE_CODE or rank > 8192:
+        w2 = self._want(w2_t, "decay matrix")
+        C = w2.shape[1]
+        if w2.shape != (rank, C) or w2.dtype not in _DTYPE_CODE or rank > 8192:
             raise KernelError(f"decay matrix {tuple(w2.shape)} does not fit a latent of {rank}")
         self._want(w0, "decay bias", torch.float32, (C,))
         out = torch.empty((N, C), dtype=torch.float32, device=self.device)

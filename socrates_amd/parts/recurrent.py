@@ -40,16 +40,17 @@ class WkvMixer:
         self.spec, self.ops = spec, ops
         self.mu = torch.stack([tensors[f"mu.{s}"] for s in _STREAMS]).contiguous()
         self.w = {s: tensors[s] for s in "rkvgo"}
-        self.w1, self.w2, self.w0 = tensors["w1"], tensors["w2"], tensors["w0"]
-        if self.w1.shape[0] != self.w2.shape[1]:
-            raise ValueError(f"wkv: the decay's two matrices do not fit ({tuple(self.w1.shape)}, {tuple(self.w2.shape)})")
+        self.w1, self.w0 = tensors["w1"], tensors["w0"]
+        if self.w1.shape[0] != tensors["w2"].shape[1]:
+            raise ValueError(f"wkv: the decay's two matrices do not fit ({tuple(self.w1.shape)}, {tuple(tensors['w2'].shape)})")
+        self.w2_t = tensors["w2"].t().contiguous()          # [rank, channels]: the kernel's threads are channels
         self.bonus, self.gain = tensors["u"], tensors["norm"]
 
     def forward(self, x, ctx, slot, write=True):
         s, ops = self.spec, self.ops
         mixes = ops.token_shift(x, self.mu, slot.state, 0, ctx)
         r, k, v, g = (ops.linear(mixes[i], self.w[name]) for i, name in enumerate("rkvg"))
-        decay = ops.wkv_decay(ops.linear(mixes[4], self.w1, out_dtype=torch.float32), self.w2, self.w0)
+        decay = ops.wkv_decay(ops.linear(mixes[4], self.w1, out_dtype=torch.float32), self.w2_t, self.w0)
         o = ops.wkv(r, k, v, decay, g, self.bonus, self.gain, s.eps, s.n_heads, slot.state, s.hidden, ctx)
         return ops.linear(o, self.w["o"])
 

@@ -84,7 +84,7 @@ def test_token_shift(kernel_sets, dtype, lengths, rows):
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_wkv_decay(kernel_sets, dtype):
     hip, ref = kernel_sets[dtype]
-    t, w2, w0 = rnd((6, 24), torch.float32, 1), rnd((200, 24), dtype, 2, 0.3), rnd((200,), torch.float32, 3)
+    t, w2, w0 = rnd((6, 24), torch.float32, 1), rnd((24, 200), dtype, 2, 0.3), rnd((200,), torch.float32, 3)
     torch.testing.assert_close(hip.wkv_decay(t, w2, w0), ref.wkv_decay(t, w2, w0), atol=1e-5, rtol=1e-4)
 
 

@@ -193,8 +193,8 @@ class TorchKernels:
             state[row, offset:offset + d] = hf[hi - 1].to(state.dtype)
         return (hf.unsqueeze(0) + (prev - hf).unsqueeze(0) * mu.to(self.acc).unsqueeze(1)).to(self.dtype)
 
-    def wkv_decay(self, t, w2, w0):
-        z = torch.tanh(t.to(self.acc)) @ w2.to(self.acc).T + w0.to(self.acc)
+    def wkv_decay(self, t, w2_t, w0):
+        z = torch.tanh(t.to(self.acc)) @ w2_t.to(self.acc) + w0.to(self.acc)
         return torch.exp(-torch.exp(z)).to(torch.float32 if self.acc == torch.float32 else self.acc)
 
     def wkv(self, r, k, v, decay, g, bonus, gain, eps, H, state, offset, ctx):
