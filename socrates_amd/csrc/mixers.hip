@@ -48,16 +48,78 @@ gated_norm_add_kernel(float* __restrict__ residual, const T* __restrict__ y, con
         out[base + c] = from_float<T>(residual[base + c] * inv * next_gain[c]);
 }
 
+// The same with the row in registers (PER elements per thread, d <= 256 * PER): every element is
+// read once, all loads are issued before the first is used.
+template <typename T, int PER>
+__global__ void __launch_bounds__(256)
+gated_norm_add_regs_kernel(float* __restrict__ residual, const T* __restrict__ y, const T* __restrict__ logits,
+                           const float* __restrict__ bias, const float* __restrict__ gain, float eps, float mult,
+                           const float* __restrict__ next_gain, float next_eps, T* __restrict__ out, int d) {
+    __shared__ float scratch[16];
+    const size_t base = (size_t)blockIdx.x * d;
+    float g[PER], res[PER], gate[PER], gn[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int c = threadIdx.x + i * 256;
+        const bool in = c < d;
+        g[i] = in ? to_float(y[base + c]) : 0.f;
+        gate[i] = (in && logits) ? to_float(logits[base + c]) + bias[c] : 0.f;
+        res[i] = in ? residual[base + c] : 0.f;
+        gn[i] = in ? gain[c] : 0.f;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        if (logits) g[i] *= soc_sigmoid(gate[i]);
+        ss += g[i] * g[i];
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = mult / sqrtf(ss / (float)d + eps);
+    float rr = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int c = threadIdx.x + i * 256;
+        res[i] += scale * gn[i] * g[i];
+        if (c < d) residual[base + c] = res[i];
+        rr += res[i] * res[i];
+    }
+    if (!next_gain) return;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int c = threadIdx.x + i * 256;
+        gn[i] = c < d ? next_gain[c] : 0.f;
+    }
+    rr = block_sum(rr, scratch);
+    const float inv = 1.f / sqrtf(rr / (float)d + next_eps);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int c = threadIdx.x + i * 256;
+        if (c < d) out[base + c] = from_float<T>(res[i] * inv * gn[i]);
+    }
+}
+
+template <typename T>
+static void launch_gated_norm_add(float* residual, const void* y, const void* logits, const float* bias, const float* gain,
+                                  float eps, float mult, const float* next_gain, float next_eps, void* out, int N, int d,
+                                  hipStream_t stream) {
+#define SOC_GNA(PER)                                                                                                    \
+    hipLaunchKernelGGL((gated_norm_add_regs_kernel<T, PER>), dim3(N), dim3(256), 0, stream, residual, (const T*)y,     \
+                       (const T*)logits, bias, gain, eps, mult, next_gain, next_eps, (T*)out, d)
+    if (d <= 1024) SOC_GNA(4);
+    else if (d <= 2048) SOC_GNA(8);
+    else if (d <= 4096) SOC_GNA(16);
+    else if (d <= 8192) SOC_GNA(32);
+    else
+        hipLaunchKernelGGL(gated_norm_add_kernel<T>, dim3(N), dim3(256), 0, stream, residual, (const T*)y, (const T*)logits,
+                           bias, gain, eps, mult, next_gain, next_eps, (T*)out, d);
+}
+
 SOC_EXPORT int soc_gated_norm_add(float* residual, const void* y, const void* logits, const float* bias,
                                   const float* gain, float eps, float mult, const float* next_gain, float next_eps,
                                   void* out, int N, int d, int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
-    if (dtype == 0)
-        hipLaunchKernelGGL(gated_norm_add_kernel<float>, dim3(N), dim3(256), 0, stream, residual, (const float*)y,
-                           (const float*)logits, bias, gain, eps, mult, next_gain, next_eps, (float*)out, d);
-    else
-        hipLaunchKernelGGL(gated_norm_add_kernel<bf16>, dim3(N), dim3(256), 0, stream, residual, (const bf16*)y,
-                           (const bf16*)logits, bias, gain, eps, mult, next_gain, next_eps, (bf16*)out, d);
+    if (dtype == 0) launch_gated_norm_add<float>(residual, y, logits, bias, gain, eps, mult, next_gain, next_eps, out, N, d, stream);
+    else launch_gated_norm_add<bf16>(residual, y, logits, bias, gain, eps, mult, next_gain, next_eps, out, N, d, stream);
     return soc_last_error();
 }
 
@@ -90,8 +152,8 @@ SOC_EXPORT int soc_glu_clamped(const void* gate_up, void* out, int N, int ff, fl
 // ---- blends of a token's input with the one before it ---------------------------------------------
 // out[s, n, c] = h[n, c] + (prev[n, c] - h[n, c]) * mu[s, c]; prev of a sequence's first token of
 // the step is what the row's state holds, which then becomes the input of its last token. Grid
-// (chunks of SHIFT_CHUNK tokens, sequences): the workgroup of a sequence's first chunk is the
-// only one that touches the state, each thread its own columns, reading before writing.
+// (chunks of SHIFT_CHUNK tokens, sequences, blocks of 256 columns): the workgroups of a sequence's
+// first chunk are the only ones that touch the state, each thread its own column, reading before writing.
 constexpr int SHIFT_CHUNK = 8;
 
 template <typename T>
@@ -105,7 +167,8 @@ token_shift_kernel(const T* __restrict__ h, const float* __restrict__ mu, int n_
     if (first >= hi) return;
     const int last = min(first + SHIFT_CHUNK, hi);
     float* kept = state + (size_t)seq_rows[seq] * stride + offset;
-    for (int c = threadIdx.x; c < d; c += blockDim.x) {
+    const int c = blockIdx.z * blockDim.x + threadIdx.x;
+    if (c < d) {
         float prev = first == lo ? kept[c] : to_float(h[(size_t)(first - 1) * d + c]);
         for (int n = first; n < last; ++n) {
             const float cur = to_float(h[(size_t)n * d + c]);
@@ -122,7 +185,8 @@ SOC_EXPORT int soc_token_shift(const void* h, const float* mu, int n_streams, fl
                                const int* seq_qstart, const int* seq_rows, void* out, int N, int d, int n_seqs,
                                int max_q_len, int dtype, hipStream_t stream) {
     if (N <= 0 || n_seqs <= 0) return 0;
-    const dim3 grid((max_q_len + SHIFT_CHUNK - 1) / SHIFT_CHUNK, n_seqs);
+    if (n_seqs > 65535 || (d + 255) / 256 > 65535) return (int)hipErrorInvalidValue;
+    const dim3 grid((max_q_len + SHIFT_CHUNK - 1) / SHIFT_CHUNK, n_seqs, (d + 255) / 256);
     if (dtype == 0)
         hipLaunchKernelGGL(token_shift_kernel<float>, grid, dim3(256), 0, stream, (const float*)h, mu, n_streams, state,
                            (size_t)stride, offset, seq_qstart, seq_rows, (float*)out, N, d);
@@ -133,17 +197,18 @@ SOC_EXPORT int soc_token_shift(const void* h, const float* mu, int n_streams, fl
 }
 
 // ---- decay = exp(-exp(tanh(t) W2^T + w0)) --------------------------------------------------------
-// t [N, rank] float32; W2 transposed, [rank, C] (consecutive threads read consecutive elements); one
-// workgroup per token keeps tanh(t) in LDS.
+// t [N, rank] float32; W2 transposed, [rank, C] (consecutive threads read consecutive elements); grid (blocks
+// of 256 channels, tokens), a thread per channel, tanh(t) of the token in LDS.
 template <typename T>
 __global__ void __launch_bounds__(256)
 wkv_decay_kernel(const float* __restrict__ t, const T* __restrict__ w2, const float* __restrict__ w0,
                  float* __restrict__ out, int C, int rank) {
     extern __shared__ float th[];
-    const int n = blockIdx.x;
+    const int n = blockIdx.y;
     for (int j = threadIdx.x; j < rank; j += blockDim.x) th[j] = tanhf(t[(size_t)n * rank + j]);
     __syncthreads();
-    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c < C) {
         float z = 0.f;
         for (int j = 0; j < rank; ++j) z = fmaf(th[j], to_float(w2[(size_t)j * C + c]), z);
         out[(size_t)n * C + c] = expf(-expf(z + w0[c]));
@@ -153,11 +218,12 @@ wkv_decay_kernel(const float* __restrict__ t, const T* __restrict__ w2, const fl
 SOC_EXPORT int soc_wkv_decay(const float* t, const void* w2, const float* w0, float* out, int N, int C, int rank,
                              int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
+    if (N > 65535) return (int)hipErrorInvalidValue;
     const size_t lds = (size_t)rank * sizeof(float);
     if (dtype == 0)
-        hipLaunchKernelGGL(wkv_decay_kernel<float>, dim3(N), dim3(256), lds, stream, t, (const float*)w2, w0, out, C, rank);
+        hipLaunchKernelGGL(wkv_decay_kernel<float>, dim3((C + 255) / 256, N), dim3(256), lds, stream, t, (const float*)w2, w0, out, C, rank);
     else
-        hipLaunchKernelGGL(wkv_decay_kernel<bf16>, dim3(N), dim3(256), lds, stream, t, (const bf16*)w2, w0, out, C, rank);
+        hipLaunchKernelGGL(wkv_decay_kernel<bf16>, dim3((C + 255) / 256, N), dim3(256), lds, stream, t, (const bf16*)w2, w0, out, C, rank);
     return soc_last_error();
 }
 
@@ -485,24 +551,28 @@ SOC_EXPORT int soc_causal_conv_silu(const void* x, int ldx, int col, int C, cons
 
 // ---- RMS norm in equal parts with a gate silu(z), in front of the norm or behind it ------------------------
 // y float32 [N, inner]; z the first `inner` columns of rows of ldz elements. Gate first: norm(y silu(z)) gain;
-// gate last: norm(y) gain silu(z). One wave per (part, token), WAVES of them in a workgroup.
-template <typename T, bool GATE_FIRST>
+// gate last: norm(y) gain silu(z). An item (part, token) is one wave's (four items to a workgroup), or, for
+// parts of 512 elements and more, a whole workgroup's.
+template <typename T, bool GATE_FIRST, int WAVES>
 __global__ void __launch_bounds__(256)
 gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, int ldz, const float* __restrict__ gain,
                         int inner, int part, int n_items, float eps, T* __restrict__ out) {
-    const int item = blockIdx.x * (blockDim.x / SOC_WAVE) + threadIdx.x / SOC_WAVE, lane = threadIdx.x % SOC_WAVE;
+    __shared__ float scratch[16];
+    constexpr int THREADS = WAVES * SOC_WAVE;
+    const int item = WAVES == 1 ? blockIdx.x * (256 / SOC_WAVE) + threadIdx.x / SOC_WAVE : blockIdx.x;
+    const int lane = threadIdx.x % THREADS;
     if (item >= n_items) return;
     const int parts = inner / part;
     const int n = item / parts, c0 = (item % parts) * part;
     float ss = 0.f;
-    for (int c = c0 + lane; c < c0 + part; c += SOC_WAVE) {
+    for (int c = c0 + lane; c < c0 + part; c += THREADS) {
         float v = y[(size_t)n * inner + c];
         if (GATE_FIRST) { const float zz = to_float(z[(size_t)n * ldz + c]); v *= zz * soc_sigmoid(zz); }
         ss += v * v;
     }
-    ss = wave_sum(ss);
+    ss = WAVES == 1 ? wave_sum(ss) : block_sum(ss, scratch);
     const float inv = 1.f / sqrtf(ss / (float)part + eps);
-    for (int c = c0 + lane; c < c0 + part; c += SOC_WAVE) {
+    for (int c = c0 + lane; c < c0 + part; c += THREADS) {
         const float zz = to_float(z[(size_t)n * ldz + c]);
         const float v = y[(size_t)n * inner + c] * zz * soc_sigmoid(zz);
         out[(size_t)n * inner + c] = from_float<T>(v * inv * gain[c]);
@@ -514,12 +584,15 @@ SOC_EXPORT int soc_gated_group_norm(const float* y, const void* z, int ldz, cons
     if (N <= 0) return 0;
     if (parts < 1 || inner % parts || (long long)N * parts > 0x7fffffffLL) return (int)hipErrorInvalidValue;
     const int items = N * parts;
-    const dim3 grid((items + 3) / 4);
-#define SOC_GGN(T, FIRST)                                                                                             \
-    hipLaunchKernelGGL((gated_group_norm_kernel<T, FIRST>), grid, dim3(256), 0, stream, y, (const T*)z, ldz, gain, inner, \
+    const bool wide = inner / parts >= 512;
+    const dim3 grid(wide ? items : (items + 3) / 4);
+#define SOC_GGN(T, FIRST, WAVES)                                                                                              \
+    hipLaunchKernelGGL((gated_group_norm_kernel<T, FIRST, WAVES>), grid, dim3(256), 0, stream, y, (const T*)z, ldz, gain, inner, \
                        inner / parts, items, eps, (T*)out)
-    if (dtype == 0) { if (gate_first) SOC_GGN(float, true); else SOC_GGN(float, false); }
-    else { if (gate_first) SOC_GGN(bf16, true); else SOC_GGN(bf16, false); }
+#define SOC_GGN_T(T)                                                                                   \
+    if (gate_first) { if (wide) SOC_GGN(T, true, 4); else SOC_GGN(T, true, 1); }                       \
+    else { if (wide) SOC_GGN(T, false, 4); else SOC_GGN(T, false, 1); }
+    if (dtype == 0) { SOC_GGN_T(float) } else { SOC_GGN_T(bf16) }
     return soc_last_error();
 }
 
