@@ -98,6 +98,79 @@ gated_norm_add_regs_kernel(float* __restrict__ residual, const T* __restrict__ y
     }
 }
 
+// The same again for widths that are multiples of 8, eight consecutive elements per load (16 bytes of
+// bfloat16, 32 of float32), CH such pieces per thread (d <= 2048 * CH); the next norm's gain comes with
+// the first loads, so the kernel waits for memory once.
+__device__ __forceinline__ void store8(float* p, const float (&x)[8]) {
+    *reinterpret_cast<float4*>(p) = make_float4(x[0], x[1], x[2], x[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(x[4], x[5], x[6], x[7]);
+}
+__device__ __forceinline__ void store8(bf16* p, const float (&x)[8]) {
+    *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]), pack_bf16x2(x[4], x[5]),
+                                              pack_bf16x2(x[6], x[7]));
+}
+
+template <typename T, int CH>
+__global__ void __launch_bounds__(256)
+gated_norm_add_vec8_kernel(float* __restrict__ residual, const T* __restrict__ y, const T* __restrict__ logits,
+                           const float* __restrict__ bias, const float* __restrict__ gain, float eps, float mult,
+                           const float* __restrict__ next_gain, float next_eps, T* __restrict__ out, int d) {
+    __shared__ float scratch[16];
+    const size_t base = (size_t)blockIdx.x * d;
+    float g[CH][8], res[CH][8], gate[CH][8], gn[CH][8], nx[CH][8];
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int c = (threadIdx.x + i * 256) * 8;
+        if (c < d) {
+            VecLoad<T, 8>::load(y + base + c, g[i]);
+            VecLoad<float, 8>::load(residual + base + c, res[i]);
+            VecLoad<float, 8>::load(gain + c, gn[i]);
+            if (logits) {
+                float b[8];
+                VecLoad<T, 8>::load(logits + base + c, gate[i]);
+                VecLoad<float, 8>::load(bias + c, b);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) gate[i][e] += b[e];
+            }
+            if (next_gain) VecLoad<float, 8>::load(next_gain + c, nx[i]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) g[i][e] = res[i][e] = gn[i][e] = gate[i][e] = nx[i][e] = 0.f;
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < CH; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if (logits) g[i][e] *= soc_sigmoid(gate[i][e]);
+            ss += g[i][e] * g[i][e];
+        }
+    ss = block_sum(ss, scratch);
+    const float scale = mult / sqrtf(ss / (float)d + eps);
+    float rr = 0.f;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int c = (threadIdx.x + i * 256) * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            res[i][e] += scale * gn[i][e] * g[i][e];
+            rr += res[i][e] * res[i][e];
+        }
+        if (c < d) store8(residual + base + c, res[i]);
+    }
+    if (!next_gain) return;
+    rr = block_sum(rr, scratch);
+    const float inv = 1.f / sqrtf(rr / (float)d + next_eps);
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int c = (threadIdx.x + i * 256) * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) res[i][e] *= inv * nx[i][e];
+        if (c < d) store8(out + base + c, res[i]);
+    }
+}
+
 template <typename T>
 static void launch_gated_norm_add(float* residual, const void* y, const void* logits, const float* bias, const float* gain,
                                   float eps, float mult, const float* next_gain, float next_eps, void* out, int N, int d,
@@ -105,7 +178,13 @@ static void launch_gated_norm_add(float* residual, const void* y, const void* lo
 #define SOC_GNA(PER)                                                                                                    \
     hipLaunchKernelGGL((gated_norm_add_regs_kernel<T, PER>), dim3(N), dim3(256), 0, stream, residual, (const T*)y,     \
                        (const T*)logits, bias, gain, eps, mult, next_gain, next_eps, (T*)out, d)
-    if (d <= 1024) SOC_GNA(4);
+#define SOC_GNA8(CH)                                                                                                    \
+    hipLaunchKernelGGL((gated_norm_add_vec8_kernel<T, CH>), dim3(N), dim3(256), 0, stream, residual, (const T*)y,      \
+                       (const T*)logits, bias, gain, eps, mult, next_gain, next_eps, (T*)out, d)
+    if (d % 8 == 0 && d <= 2048) SOC_GNA8(1);
+    else if (d % 8 == 0 && d <= 4096) SOC_GNA8(2);
+    else if (d % 8 == 0 && d <= 8192) SOC_GNA8(4);
+    else if (d <= 1024) SOC_GNA(4);
     else if (d <= 2048) SOC_GNA(8);
     else if (d <= 4096) SOC_GNA(16);
     else if (d <= 8192) SOC_GNA(32);

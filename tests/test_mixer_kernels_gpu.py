@@ -47,7 +47,8 @@ STEPS = [([1], [0]), ([2, 1, 37], [3, 0, 5]), ([70, 1, 1, 9], [1, 6, 2, 4])]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("N,d,gated,follows", [(1, 64, True, True), (9, 72, True, False), (5, 2560, False, True), (3, 1000, True, True)])
+@pytest.mark.parametrize("N,d,gated,follows", [(1, 64, True, True), (9, 72, True, False), (5, 2560, False, True), (3, 1001, True, True), (2, 4100, True, False),
+                                                (2, 8192, True, True), (2, 9001, True, True)])
 def test_gated_norm_add(kernel_sets, dtype, N, d, gated, follows):
     hip, ref = kernel_sets[dtype]
     res, y = rnd((N, d), torch.float32, 1), rnd((N, d), dtype, 2, 0.3)
