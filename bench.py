@@ -261,8 +261,8 @@ def mitisun_dict(width, ff, n_layers, wkv_heads, ssm_heads, attn_heads, window=1
 
 def mitisun_beside_qwen3(args, dtype, item):
     """Prefill and decode of Mitisun at a few real layer sizes, each beside Qwen3 of the same width,
-    feed-forward size, vocabulary and number of layers. One JSON line of its own; the default
-    workload's line and contract are untouched."""
+    feed-forward size, vocabulary and number of layers, both with the library's default solutions for its
+    products (no tuning pass). One JSON line of its own; the default workload's line and contract are untouched."""
     import torch
     sizes = [("4b", "qwen3-4b", dict(wkv_heads=40, ssm_heads=80, attn_heads=20)),
              ("8b", "qwen3-8b", dict(wkv_heads=64, ssm_heads=128, attn_heads=32))]
@@ -280,8 +280,7 @@ def mitisun_beside_qwen3(args, dtype, item):
             config, engine = build_engine(cfg, dtype, args.batch, args.max_len, seed=0, compile_=not args.no_graphs,
                                           chunk=max(2048, args.prefill_tokens), block_size=args.block_size)
             V = cfg.get("vocab_size") or cfg["vocab"]
-            if args.dtype == "bf16" and not args.no_tune:
-                engine.tune([args.prefill_tokens, args.batch])
+            # (no tuning pass here, for either model: both run the library's default solutions)
             tok_s, ms = decode_rate(engine, args.batch, args.context, args.steps, args.warmup, V, seed=1)
             pre_s = prefill_rate(engine, args.prefill_tokens, V, seed=2)
             weights = config.param_counts()["read_per_step"] * item

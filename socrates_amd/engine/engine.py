@@ -225,6 +225,12 @@ class Engine:
         ops = self.runner.ops
         if not hasattr(ops, "library_tuning"):
             return
+        if any(getattr(b, "library_tuning", True) is False for b in self.runner.model.blocks):
+            # a block arrangement whose models the tuning pass has aborted on: its products keep the
+            # library's default choices
+            import warnings
+            warnings.warn("tune(): skipped, a block of this model declares library_tuning = False", stacklevel=2)
+            return
         if token_counts is None:
             token_counts = [self.scheduler.token_budget, self.max_batch]
         kept = (self.n_steps, self.prompt_tokens, self.output_tokens)

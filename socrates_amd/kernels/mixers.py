@@ -200,10 +200,13 @@ class Mixers:
         if out.dim() != 3 or out.shape[:2] != (N, H) or out.shape[2] < n_out:
             raise KernelError(f"per-head product: out {tuple(out.shape)}")
         if (self.dtype == torch.bfloat16 and N > 16 and self.library_gemm and K % 8 == 0 and n_out % 8 == 0
-                and not torch.cuda.is_current_stream_capturing()):
+                and not self._tuning and not torch.cuda.is_current_stream_capturing()):
             # more than 16 rows in bfloat16: the library's batched product, as for every other
-            # product of that size (float32 sums inside); its [H, N, n_out] result is laid back by head
-            out[:, :, :n_out].copy_(torch.bmm(x.transpose(0, 1)[:, :, :K], w.transpose(1, 2)).transpose(0, 1))
+            # product of that size (float32 sums inside), from operands laid out by head (never while the
+            # library times its solutions: its tuning pass is kept to plain products); its [H, N, n_out]
+            # result is laid back by head
+            by_head = x.transpose(0, 1)[:, :, :K].contiguous()
+            out[:, :, :n_out].copy_(torch.bmm(by_head, w.transpose(1, 2)).transpose(0, 1))
             return out
         _check(self._mixers().soc_head_linear(_ptr(x), c_int(ldx), _ptr(w), _ptr(out), c_int(out.shape[2]), c_int(N), c_int(H),
                                               c_int(n_out), c_int(K), c_int(self.code), self._stream()), "head_linear")

@@ -120,6 +120,10 @@ class SandwichBlock:
     norm of the branch's result, the scaled sum into the stream, and the norm that opens the
     next branch (this block's second, or the next block's first)."""
     chains = True
+    # ``Engine.tune`` leaves models with such blocks alone: the one run of the library's tuning pass over
+    # such a model (4B-sized layers, a prompt of 2,048 tokens) aborted on the GPU and the cause is not
+    # known; every product keeps the library's default solution.
+    library_tuning = False
 
     def __init__(self, spec: BlockSpec, weights, ops):
         self.spec, self.ops = spec, ops
