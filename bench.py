@@ -262,7 +262,7 @@ def mitisun_dict(width, ff, n_layers, wkv_heads, ssm_heads, attn_heads, window=1
 def mitisun_beside_qwen3(args, dtype, item):
     """Prefill and decode of Mitisun at a few real layer sizes, each beside Qwen3 of the same width,
     feed-forward size, vocabulary and number of layers, both with the library's default solutions for its
-    products (no tuning pass). One JSON line of its own; the default workload's line and contract are untouched."""
+    products (no tuning pass). One JSON line of its own; the default workload and its line are untouched."""
     import torch
     sizes = [("4b", "qwen3-4b", dict(wkv_heads=40, ssm_heads=80, attn_heads=20)),
              ("8b", "qwen3-8b", dict(wkv_heads=64, ssm_heads=128, attn_heads=32))]
