@@ -15,6 +15,16 @@
 
 __device__ __forceinline__ float soc_sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
 
+__device__ __forceinline__ void store8(float* p, const float (&x)[8]) {
+    *reinterpret_cast<float4*>(p) = make_float4(x[0], x[1], x[2], x[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(x[4], x[5], x[6], x[7]);
+}
+__device__ __forceinline__ void store8(bf16* p, const float (&x)[8]) {
+    *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]), pack_bf16x2(x[4], x[5]),
+                                              pack_bf16x2(x[6], x[7]));
+}
+
+
 // ---- the close of a branch ---------------------------------------------------------------------
 // residual += mult * gain * g / rms(g) with g = y * sigmoid(logits + bias) (no gate: g = y);
 // then, if next_gain is given, out = residual / rms(residual) * next_gain.
@@ -101,15 +111,6 @@ gated_norm_add_regs_kernel(float* __restrict__ residual, const T* __restrict__ y
 // The same again for widths that are multiples of 8, eight consecutive elements per load (16 bytes of
 // bfloat16, 32 of float32), CH such pieces per thread (d <= 2048 * CH); the next norm's gain comes with
 // the first loads, so the kernel waits for memory once.
-__device__ __forceinline__ void store8(float* p, const float (&x)[8]) {
-    *reinterpret_cast<float4*>(p) = make_float4(x[0], x[1], x[2], x[3]);
-    *reinterpret_cast<float4*>(p + 4) = make_float4(x[4], x[5], x[6], x[7]);
-}
-__device__ __forceinline__ void store8(bf16* p, const float (&x)[8]) {
-    *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf16x2(x[0], x[1]), pack_bf16x2(x[2], x[3]), pack_bf16x2(x[4], x[5]),
-                                              pack_bf16x2(x[6], x[7]));
-}
-
 template <typename T, int CH>
 __global__ void __launch_bounds__(256)
 gated_norm_add_vec8_kernel(float* __restrict__ residual, const T* __restrict__ y, const T* __restrict__ logits,
@@ -214,10 +215,40 @@ __global__ void glu_clamped_kernel(const T* __restrict__ gate_up, T* __restrict_
     out[i] = from_float<T>(g * soc_sigmoid(slope * g) * (u + 1.f));
 }
 
+// (eight consecutive elements per lane where ff is a multiple of 8)
+template <typename T>
+__global__ void glu_clamped_vec8_kernel(const T* __restrict__ gate_up, T* __restrict__ out, size_t groups, int ff,
+                                        float limit, float slope) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= groups) return;
+    const int per_row = ff / 8;
+    const size_t n = i / per_row, c = (i % per_row) * 8;
+    float g[8], u[8], y[8];
+    VecLoad<T, 8>::load(gate_up + n * 2 * ff + c, g);
+    VecLoad<T, 8>::load(gate_up + n * 2 * ff + ff + c, u);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float gg = fminf(g[e], limit), uu = fminf(fmaxf(u[e], -limit), limit);
+        y[e] = gg * soc_sigmoid(slope * gg) * (uu + 1.f);
+    }
+    store8(out + n * ff + c, y);
+}
+
 SOC_EXPORT int soc_glu_clamped(const void* gate_up, void* out, int N, int ff, float limit, float slope, int dtype,
                                hipStream_t stream) {
     const size_t total = (size_t)N * ff;
     if (total == 0) return 0;
+    if (ff % 8 == 0) {
+        const size_t groups = total / 8;
+        const dim3 grid((unsigned)((groups + 255) / 256));
+        if (dtype == 0)
+            hipLaunchKernelGGL(glu_clamped_vec8_kernel<float>, grid, dim3(256), 0, stream, (const float*)gate_up, (float*)out,
+                               groups, ff, limit, slope);
+        else
+            hipLaunchKernelGGL(glu_clamped_vec8_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)gate_up, (bf16*)out,
+                               groups, ff, limit, slope);
+        return soc_last_error();
+    }
     const dim3 grid((unsigned)((total + 255) / 256));
     if (dtype == 0)
         hipLaunchKernelGGL(glu_clamped_kernel<float>, grid, dim3(256), 0, stream, (const float*)gate_up, (float*)out,

@@ -66,8 +66,9 @@ def test_gated_norm_add(kernel_sets, dtype, N, d, gated, follows):
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_glu_clamped(kernel_sets, dtype):
     hip, ref = kernel_sets[dtype]
-    x = rnd((7, 2 * 93), dtype, 1, 2.0)
-    close(hip.glu_clamped(x, 1.5, 1.702), ref.glu_clamped(x, 1.5, 1.702), dtype)
+    for ff in (93, 96, 1000):
+        x = rnd((7, 2 * ff), dtype, 1, 2.0)
+        close(hip.glu_clamped(x, 1.5, 1.702), ref.glu_clamped(x, 1.5, 1.702), dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -136,6 +137,39 @@ def test_ssd(kernel_sets, dtype, lengths, rows, H, P, Ns, G):
     assert a.dtype == torch.float32
     torch.testing.assert_close(a, b, atol=2e-4, rtol=2e-4)
     torch.testing.assert_close(s1, s2, atol=1e-4, rtol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("size", [16, 24, 48, 64, 96, 128, 192, 256])
+@pytest.mark.parametrize("seqs", [2, 12])
+def test_recurrences_at_every_state_size(kernel_sets, dtype, size, seqs):
+    """Every size the kernels are built for, with few workgroups (a head's columns in blocks of 16) and with
+    many (blocks of 64): 24 heads, sequences of one to nine tokens, from a non-zero state."""
+    hip, ref = kernel_sets[dtype]
+    H = 24
+    lengths = [1 + (3 * i) % 9 for i in range(seqs)]
+    ctx = step_of(lengths, list(range(seqs)))
+    N = ctx.n_tokens
+    # wkv: keys and columns of `size`
+    C = H * size
+    r, k, v, g = (rnd((N, C), dtype, i, 0.5) for i in range(4))
+    decay = torch.rand((N, C), generator=torch.Generator().manual_seed(9)).to(DEV) * 0.5 + 0.5
+    bonus, gain = rnd((H, size), torch.float32, 5), rnd((C,), torch.float32, 6)
+    s1 = rnd((seqs, H * size * size), torch.float32, 7)
+    s2 = s1.clone()
+    close(hip.wkv(r, k, v, decay, g, bonus, gain, 1e-5, H, s1, 0, ctx), ref.wkv(r, k, v, decay, g, bonus, gain, 1e-5, H, s2, 0, ctx),
+          dtype, atol=5e-4 if dtype == torch.float32 else 3e-2)
+    torch.testing.assert_close(s1, s2, atol=2e-4, rtol=2e-4)
+    # ssd: a state of `size` keys, 40 columns, heads in 3 groups
+    P, G = 40, 3
+    xbc, dt = rnd((N, H * P + 2 * G * size), dtype, 11, 0.5), rnd((N, H), torch.float32, 12)
+    dt_bias, a_log, skip = rnd((H,), torch.float32, 13), rnd((H,), torch.float32, 14, 0.5), rnd((H,), torch.float32, 15)
+    s1 = rnd((seqs, H * size * P), torch.float32, 16)
+    s2 = s1.clone()
+    a = hip.ssd(xbc, dt, dt_bias, a_log, skip, H, P, size, G, s1, 0, ctx)
+    b = ref.ssd(xbc, dt, dt_bias, a_log, skip, H, P, size, G, s2, 0, ctx)
+    torch.testing.assert_close(a, b, atol=5e-4, rtol=5e-4)
+    torch.testing.assert_close(s1, s2, atol=2e-4, rtol=2e-4)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
