@@ -492,7 +492,7 @@ ssd_kernel(const T* __restrict__ xbc, const float* __restrict__ dt_raw, const fl
            float* __restrict__ state, size_t stride, int offset, const int* __restrict__ seq_qstart,
            const int* __restrict__ seq_rows, float* __restrict__ out) {
     constexpr int REC_TB = rec_batch(NK), PARTS = 256 / CW, KPT = NK / PARTS, STAGE = (REC_TB * NK + 255) / 256;
-    __shared__ float sb[2][REC_TB][NK], sc[2][REC_TB][NK], skeep[2][REC_TB];
+    __shared__ float sb[2][REC_TB][NK], sc[2][REC_TB][NK], skeep[2][REC_TB], sdt[2][REC_TB];
     __shared__ float red[REC_TB][PARTS][CW];
     const int blocks = (P + CW - 1) / CW;
     const int head = blockIdx.x / blocks, seq = blockIdx.y, tid = threadIdx.x;
@@ -514,7 +514,8 @@ ssd_kernel(const T* __restrict__ xbc, const float* __restrict__ dt_raw, const fl
         return z > 20.f ? z : log1pf(expf(z));
     };
 
-    float fb[STAGE], fc[STAGE], fx[REC_TB], fkeep = 0.f;
+    // (a token's step size and decay are computed once, by one thread, and go through LDS with B and C)
+    float fb[STAGE], fc[STAGE], fx[REC_TB], fdt = 0.f, fkeep = 1.f;
     auto fetch = [&](int n0) {
 #pragma unroll
         for (int t = 0; t < REC_TB; ++t)
@@ -524,10 +525,13 @@ ssd_kernel(const T* __restrict__ xbc, const float* __restrict__ dt_raw, const fl
             const int e = tid + q * 256, t = e / NK, i = e % NK;
             const bool in = t < REC_TB && n0 + t < hi && i < Ns;
             const T* row = xbc + (size_t)(n0 + t) * ld;
-            fb[q] = in ? step_size(n0 + t) * to_float(row[boff + i]) : 0.f;
+            fb[q] = in ? to_float(row[boff + i]) : 0.f;
             fc[q] = in ? to_float(row[coff + i]) : 0.f;
         }
-        if (tid < REC_TB) fkeep = n0 + tid < hi ? expf(-rate * step_size(n0 + tid)) : 1.f;
+        if (tid < REC_TB) {
+            fdt = n0 + tid < hi ? step_size(n0 + tid) : 0.f;
+            fkeep = expf(-rate * fdt);
+        }
     };
     auto land = [&](int buf) {
 #pragma unroll
@@ -535,7 +539,7 @@ ssd_kernel(const T* __restrict__ xbc, const float* __restrict__ dt_raw, const fl
             const int e = tid + q * 256, t = e / NK, i = e % NK;
             if (t < REC_TB) { sb[buf][t][i] = fb[q]; sc[buf][t][i] = fc[q]; }
         }
-        if (tid < REC_TB) skeep[buf][tid] = fkeep;
+        if (tid < REC_TB) { sdt[buf][tid] = fdt; skeep[buf][tid] = fkeep; }
     };
     fetch(lo);
     land(0);
@@ -551,11 +555,11 @@ ssd_kernel(const T* __restrict__ xbc, const float* __restrict__ dt_raw, const fl
 #pragma unroll
         for (int t = 0; t < REC_TB; ++t) {
             if (t < nb) {
-                const float keep = skeep[buf][t];
+                const float keep = skeep[buf][t], dx = sdt[buf][t] * xj[t];
                 float acc = part == 0 ? through * xj[t] : 0.f;
 #pragma unroll
                 for (int ii = 0; ii < KPT; ++ii) {
-                    s[ii] = fmaf(keep, s[ii], sb[buf][t][i0 + ii] * xj[t]);
+                    s[ii] = fmaf(keep, s[ii], sb[buf][t][i0 + ii] * dx);
                     acc = fmaf(sc[buf][t][i0 + ii], s[ii], acc);
                 }
                 red[t][part][tid % CW] = acc;
