@@ -141,13 +141,13 @@ def test_ssd(kernel_sets, dtype, lengths, rows, H, P, Ns, G):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("size", [16, 24, 48, 64, 96, 128, 192, 256])
-@pytest.mark.parametrize("seqs", [2, 12])
-def test_recurrences_at_every_state_size(kernel_sets, dtype, size, seqs):
-    """Every size the kernels are built for, with few workgroups (a head's columns in blocks of 16) and with
-    many (blocks of 64): 24 heads, sequences of one to nine tokens, from a non-zero state."""
+@pytest.mark.parametrize("seqs,H,longest", [(2, 24, 9), (12, 24, 9), (2, 24, 70), (2, 5, 70)])
+def test_recurrences_at_every_state_size(kernel_sets, dtype, size, seqs, H, longest):
+    """Every size the kernels are built for, in both layouts of a head's columns over workgroups: blocks of 16
+    (few heads and sequences, or a prompt portion in the step) and of 64 (many single tokens); sequences of one
+    token to ``longest``, from a non-zero state."""
     hip, ref = kernel_sets[dtype]
-    H = 24
-    lengths = [1 + (3 * i) % 9 for i in range(seqs)]
+    lengths = [1 + (3 * i) % 9 for i in range(seqs - 1)] + [longest]
     ctx = step_of(lengths, list(range(seqs)))
     N = ctx.n_tokens
     # wkv: keys and columns of `size`
@@ -161,7 +161,7 @@ def test_recurrences_at_every_state_size(kernel_sets, dtype, size, seqs):
           dtype, atol=5e-4 if dtype == torch.float32 else 3e-2)
     torch.testing.assert_close(s1, s2, atol=2e-4, rtol=2e-4)
     # ssd: a state of `size` keys, 40 columns, heads in 3 groups
-    P, G = 40, 3
+    P, G = 40, (3 if H % 3 == 0 else 1)
     xbc, dt = rnd((N, H * P + 2 * G * size), dtype, 11, 0.5), rnd((N, H), torch.float32, 12)
     dt_bias, a_log, skip = rnd((H,), torch.float32, 13), rnd((H,), torch.float32, 14, 0.5), rnd((H,), torch.float32, 15)
     s1 = rnd((seqs, H * size * P), torch.float32, 16)
