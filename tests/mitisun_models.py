@@ -51,7 +51,7 @@ MIX_A = model(64, 97, [mamba2(4, 16, 16, groups=2, conv=3, norm_groups=2),
                        latent(3, 16, 8, 24, 24, 20, window=9, scale=0.9),
                        wkv(2, 32),
                        latent(3, 16, 8, 24, 24, 36, window=5, scale=1.2, kv_from=1),
-                       wkv(4, 16)], ff=96, limit=1.0, mult=0.5, no_ff=(2,))
+                       wkv(3, 16)], ff=96, limit=1.0, mult=0.5, no_ff=(2,))
 MIX_B = model(96, 130, [wkv(4, 24),
                         latent(2, 40, 12, 40, 52, 30, window=200, base=500.0, dims=8),
                         mamba2(6, 16, 20, groups=1, conv=2, norm_groups=1),
@@ -59,6 +59,46 @@ MIX_B = model(96, 130, [wkv(4, 24),
               ff=200, limit=3.0, mult=1.0, eps=3e-6)
 MODELS = {"wkv": ONE_WKV, "mamba2": ONE_MAMBA, "latent": ONE_LATENT, "A": MIX_A, "B": MIX_B}
 BLOCK = {"wkv": 16, "mamba2": 16, "latent": 4, "A": 4, "B": 16}
+
+
+def drawn_model(seed):
+    """A configuration drawn from everything config.json can say: 2 to 6 layers in any order, sizes that are
+    no multiples of anything, windows of one token up to longer than the prompts, one to five taps, a layer
+    now and then without feed-forward, attention layers that read an earlier one's cache."""
+    import random
+    rng = random.Random(seed)
+    width = rng.choice([24, 40, 56, 64, 88, 128])
+    layers, writers, no_ff = [], [], []
+    for i in range(rng.randint(2, 6)):
+        kind = rng.choice(["wkv", "mamba2", "latent", "latent"])
+        if kind == "wkv":
+            layers.append(wkv(rng.randint(1, 5), rng.choice([8, 12, 16, 24, 40, 64])))
+            layers[-1]["mixer"]["decay_rank"] = rng.choice([1, 3, 8, 20])
+        elif kind == "mamba2":
+            groups = rng.choice([1, 2, 3])
+            layers.append(mamba2(groups * rng.randint(1, 3), rng.choice([4, 8, 20, 32]), rng.choice([4, 8, 16, 24, 40, 64]),
+                                 groups=groups, conv=rng.randint(1, 5), norm_groups=1))
+            m = layers[-1]["mixer"]
+            m["norm_groups"] = rng.choice([g for g in (1, 2, 3, 4) if (m["heads"] * m["vdim"]) % g == 0])
+        else:
+            window = rng.choice([1, 2, 5, 17, 64, 300])
+            if writers and rng.random() < 0.5:
+                j = rng.choice(writers)
+                src = layers[j]["mixer"]
+                layers.append(latent(rng.randint(1, 6), rng.choice([4, 8, 16, 24, 48]), src["rot_dim"], rng.choice([4, 8, 20, 32]),
+                                     src["kv_rank"], rng.choice([4, 12, 32]), window, base=src["rot"]["base"],
+                                     scale=rng.choice([0.3, 1.0, 2.5]), kv_from=j, dims=src["rot"]["dims"]))
+            else:
+                rot_dim = rng.choice([2, 4, 6, 8, 16, 32])
+                layers.append(latent(rng.randint(1, 6), rng.choice([4, 8, 16, 24, 48]), rot_dim, rng.choice([4, 8, 20, 32]),
+                                     rng.choice([8, 12, 24, 40, 64, 100]), rng.choice([4, 12, 32]), window,
+                                     base=rng.choice([100.0, 10000.0, 250000.0]), scale=rng.choice([0.3, 1.0, 2.5]),
+                                     dims=rng.choice([d for d in (2, 4, 6, 8, 16, 32) if d <= rot_dim])))
+                writers.append(i)
+        if rng.random() < 0.2:
+            no_ff.append(i)
+    return model(width, rng.choice([37, 64, 101]), layers, ff=rng.choice([24, 50, 96]), limit=rng.choice([0.5, 2.0, 6.0]),
+                 mult=rng.choice([0.3, 0.7, 1.0]), eps=rng.choice([1e-6, 1e-5, 1e-3]), no_ff=tuple(no_ff))
 
 
 def tensor_shapes(cfg):
@@ -129,6 +169,14 @@ def write_model(folder, cfg, seed, weights=None):
 def oracle(folder, prompts):
     cfg, w = plain.read_folder(folder, torch.float64)
     return [plain.forward(cfg, w, p).float() for p in prompts]
+
+
+def row_errors(got, want):
+    """Per row: the difference of the logits, mean taken off, root mean square over the vocabulary, in units of
+    the row's spread."""
+    got, want = got.double(), want.double()
+    d = (got - got.mean(-1, keepdim=True)) - (want - want.mean(-1, keepdim=True))
+    return d.pow(2).mean(-1).sqrt() / want.std(-1)
 
 
 def compare(got, want, tol, what=""):

@@ -11,7 +11,7 @@ import torch
 
 import plain_mitisun as plain
 from helpers import random_prompts, replay, make_runner
-from mitisun_models import BLOCK, CUTS, MODELS, check_trace, compare, latent, model, oracle, random_weights, write_model, wkv, mamba2
+from mitisun_models import BLOCK, CUTS, MODELS, check_trace, compare, drawn_model, latent, model, oracle, random_weights, write_model, wkv, mamba2
 from socrates_amd.config import ConfigError, MitisunConfig, load_config
 from socrates_amd.engine import StepEntry
 from socrates_amd.parts import cache_needs, expected_tensors
@@ -160,6 +160,35 @@ def test_pages_behind_the_window_come_back(folders):
     prompts = random_prompts([100], cfg["vocab"], seed=24)
     # 100 tokens in pages of 4 would be 25 pages; a portion of up to 33 tokens behind a window of 9 needs 12
     check_trace(folders["A"], ops32(), prompts, CUTS["portions"](prompts), TOL, block_size=4, num_blocks=12, max_len=128)
+
+
+def test_a_token_far_back_reaches_through_the_states(tmp_path):
+    """Slow decays (a state that forgets a hundredth per token) and no attention: what the first token was still
+    shows 150 tokens later, in the plain model by far more than the tolerance, and the framework carries it
+    through portions of every size and through single tokens."""
+    cfg = model(48, 50, [wkv(2, 24), mamba2(3, 16, 12, conv=2)], mult=1.0)
+    w = random_weights(cfg, 31)
+    w["l0.mix.w0"] = torch.full_like(w["l0.mix.w0"], -4.6)          # decay exp(-exp(-4.6)) = 0.99
+    w["l1.mix.A_log"] = torch.full_like(w["l1.mix.A_log"], -2.3)    # rate 0.1 ...
+    w["l1.mix.dt_bias"] = torch.full_like(w["l1.mix.dt_bias"], -2.2)  # ... times steps of about 0.1
+    folder = write_model(tmp_path / "m", cfg, 31, w)
+    prompt = random_prompts([160], cfg["vocab"], seed=32)[0]
+    other = [(prompt[0] + 7) % cfg["vocab"]] + prompt[1:]
+    want, moved = oracle(folder, [prompt, other])
+    with pytest.raises(AssertionError):
+        compare(moved[150:], want[150:], 50 * TOL)
+    for cut in ("portions", "tail"):
+        check_trace(folder, ops32(), [prompt], CUTS[cut]([prompt]), TOL, want=[want], max_len=192, what=f"far {cut}")
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_drawn_configurations(tmp_path, seed):
+    cfg = drawn_model(seed)
+    folder = write_model(tmp_path / "m", cfg, seed=100 + seed)
+    prompts = random_prompts([23, 1, 40, 9], cfg["vocab"], seed=seed)
+    block = [2, 4, 16][seed % 3]
+    check_trace(folder, ops32(), prompts, CUTS[["mixed", "portions", "tail"][seed % 3]](prompts), TOL, block_size=block,
+                max_len=64, what=f"drawn {seed}")
 
 
 def test_long_decoding(folders):

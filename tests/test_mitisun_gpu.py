@@ -15,7 +15,7 @@ import torch
 
 import plain_mitisun as plain
 from helpers import make_runner, random_prompts, replay, trace_mixed, trace_tail_decode
-from mitisun_models import BLOCK, CUTS, MODELS, check_trace, compare, latent, mamba2, model, oracle, wkv, write_model
+from mitisun_models import BLOCK, CUTS, MODELS, check_trace, compare, drawn_model, row_errors, latent, mamba2, model, oracle, wkv, write_model
 
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parents[1]
@@ -46,6 +46,38 @@ def test_cuts_match_the_plain_model(folders, kernel_sets, name, cut, dtype):
     pool = dict(num_blocks=4 * (-(-72 // BLOCK[name]))) if cut == "mixed" else {}
     check_trace(folders[name], kernel_sets[dtype], prompts, CUTS[cut](prompts), TOL[dtype], block_size=BLOCK[name], max_len=128,
                 what=f"{name} {cut} {dtype}", **pool)
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
+@pytest.mark.parametrize("seed", range(24))
+def test_drawn_configurations(tmp_path, kernel_sets, seed, dtype):
+    """Configurations drawn from everything config.json can say (layer order, every size, windows of one token
+    and longer than the prompts, one to five taps, shared caches, layers without feed-forward), each under one
+    way of cutting its requests, captured decode steps included. Such models can be touchy (a width of 24, a
+    sharp softmax, a large eps): in bfloat16 a request is judged against what rounding alone does to it, which
+    the stand-in kernels in bfloat16 on the CPU say (they round where the HIP kernels round): within three times
+    that, per request, for the worst row and for nine rows in ten."""
+    cfg = drawn_model(seed)
+    folder = write_model(tmp_path / "m", cfg, seed=100 + seed)
+    prompts = random_prompts([23, 1, 40, 9], cfg["vocab"], seed=seed)
+    block = [2, 4, 16][seed % 3]
+    runner = make_runner(folder, kernel_sets[dtype], max_rows=4, max_len=64, block_size=block)
+    if seed % 2:
+        runner.enable_graphs(4)
+    got = replay(runner, CUTS[["mixed", "portions", "tail"][seed % 3]](prompts))
+    want = oracle(folder, prompts)
+    if dtype == "float32":
+        for i in range(len(prompts)):
+            compare(got[f"r{i}"], want[i], TOL[dtype], f"drawn {seed} {dtype} request {i}")
+        return
+    from torch_kernels import TorchKernels
+    rounded = replay(make_runner(folder, TorchKernels(torch.bfloat16, "cpu"), max_rows=4, max_len=64, block_size=block),
+                     CUTS[["mixed", "portions", "tail"][seed % 3]](prompts))
+    for i in range(len(prompts)):
+        mine, noise = row_errors(got[f"r{i}"], want[i]), row_errors(rounded[f"r{i}"], want[i])
+        nine = max(1, int(0.9 * mine.numel()))
+        assert float(mine.max()) <= 3 * float(noise.max()) + 0.03, f"drawn {seed} request {i}: {float(mine.max()):.3g} against {float(noise.max()):.3g}"
+        assert float(mine.kthvalue(nine).values) <= 3 * float(noise.kthvalue(nine).values) + 0.03, f"drawn {seed} request {i}, nine rows in ten"
 
 
 @pytest.mark.parametrize("dtype", list(DTYPES))
