@@ -81,6 +81,19 @@ def test_drawn_configurations(tmp_path, kernel_sets, seed, dtype):
 
 
 @pytest.mark.parametrize("dtype", list(DTYPES))
+@pytest.mark.parametrize("heads", [17, 20, 33])
+def test_many_heads_on_one_cached_vector(tmp_path, kernel_sets, heads, dtype):
+    """All heads of a latent-attention layer share one cached vector, one "kv head" for the attention kernels:
+    more than sixteen of them, which is more than one row block of the MFMA kernels per token."""
+    cfg = model(64, 60, [latent(heads, 8, 8, 8, 24, 16, window=21, scale=0.8), wkv(2, 16)], mult=0.7)
+    folder = write_model(tmp_path / "m", cfg, seed=60 + heads)
+    prompts = random_prompts([50, 3, 33], cfg["vocab"], seed=heads)
+    for cut in ("whole", "tail", "mixed"):
+        check_trace(folder, kernel_sets[dtype], prompts, CUTS[cut](prompts), TOL[dtype], block_size=16, max_len=64,
+                    what=f"{heads} heads {cut} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
 def test_window_edges_and_long_decoding(tmp_path, kernel_sets, dtype):
     """A window of 6 (in float32 under a sharp softmax, so the key at the edge often carries the weight;
     in bfloat16 a flat one, where every key of six counts and rounding moves little), pages of 4, 150
