@@ -835,10 +835,47 @@ head_linear_kernel(const T* __restrict__ x, int ldx, const T* __restrict__ w, T*
                 out[((size_t)(n0 + tn * 4 + t) * H + head) * ldo + o0 + to] = from_float<T>(acc[t]);
 }
 
+// The same product for steps of at most 16 tokens, where the tiles above would wait for memory once per 32 k:
+// a wave per (head, output), its lanes over k, all loads issued at once, one sum over the wave per token.
+template <typename T>
+__global__ void __launch_bounds__(256)
+head_linear_rows_kernel(const T* __restrict__ x, int ldx, const T* __restrict__ w, T* __restrict__ out, int ldo,
+                        int N, int H, int n_out, int K) {
+    const int head = blockIdx.y, o = blockIdx.x * 4 + threadIdx.x / SOC_WAVE, lane = threadIdx.x % SOC_WAVE;
+    if (o >= n_out) return;
+    float acc[16];
+#pragma unroll
+    for (int n = 0; n < 16; ++n) acc[n] = 0.f;
+    const T* wrow = w + ((size_t)head * n_out + o) * K;
+    for (int k = lane; k < K; k += SOC_WAVE) {
+        const float wv = to_float(wrow[k]);
+#pragma unroll
+        for (int n = 0; n < 16; ++n)
+            if (n < N) acc[n] = fmaf(to_float(x[((size_t)n * H + head) * ldx + k]), wv, acc[n]);
+    }
+#pragma unroll
+    for (int n = 0; n < 16; ++n) {
+        if (n < N) {
+            const float sum = wave_sum(acc[n]);
+            if (lane == 0) out[((size_t)n * H + head) * ldo + o] = from_float<T>(sum);
+        }
+    }
+}
+
 SOC_EXPORT int soc_head_linear(const void* x, int ldx, const void* w, void* out, int ldo, int N, int H, int n_out, int K,
                                int dtype, hipStream_t stream) {
     if (N <= 0 || H <= 0 || n_out <= 0) return 0;
     if (K < 1 || K > ldx || n_out > ldo || H > 65535 || (N + 15) / 16 > 65535) return (int)hipErrorInvalidValue;
+    if (N <= 16) {
+        const dim3 rows_grid((n_out + 3) / 4, H);
+        if (dtype == 0)
+            hipLaunchKernelGGL(head_linear_rows_kernel<float>, rows_grid, dim3(256), 0, stream, (const float*)x, ldx,
+                               (const float*)w, (float*)out, ldo, N, H, n_out, K);
+        else
+            hipLaunchKernelGGL(head_linear_rows_kernel<bf16>, rows_grid, dim3(256), 0, stream, (const bf16*)x, ldx,
+                               (const bf16*)w, (bf16*)out, ldo, N, H, n_out, K);
+        return soc_last_error();
+    }
     const dim3 grid((n_out + 63) / 64, (N + 15) / 16, H);
     if (dtype == 0)
         hipLaunchKernelGGL(head_linear_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, ldx, (const float*)w,

@@ -206,7 +206,8 @@ def test_latent_write_and_query(kernel_sets, dtype, R, Dr, dims, width, block):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("N,H,ldx,K,n_out", [(1, 1, 16, 16, 16), (19, 5, 80, 64, 70), (70, 2, 144, 100, 129)])
+@pytest.mark.parametrize("N,H,ldx,K,n_out", [(1, 1, 16, 16, 16), (8, 20, 160, 128, 96), (16, 3, 80, 70, 33), (17, 3, 80, 70, 33), (19, 5, 80, 64, 70),
+                                             (70, 2, 144, 100, 129)])
 def test_head_project(kernel_sets, dtype, N, H, ldx, K, n_out):
     hip, ref = kernel_sets[dtype]
     x, w = rnd((N, H, ldx), dtype, 1), rnd((H, n_out, K), dtype, 2, 0.2)
