@@ -26,19 +26,20 @@ __device__ __forceinline__ void store8(bf16* p, const float (&x)[8]) {
 
 
 // ---- the close of a branch ---------------------------------------------------------------------
-// residual += mult * gain * g / rms(g) with g = y * sigmoid(logits + bias) (no gate: g = y);
+// residual += mult * gain * g / rms(g) with g = y * sigmoid(logits + bias) (no gate: g = y); the logits are the
+// first d elements of rows of ldg elements (they may be columns of a wider product);
 // then, if next_gain is given, out = residual / rms(residual) * next_gain.
 template <typename T>
 __global__ void __launch_bounds__(256)
-gated_norm_add_kernel(float* __restrict__ residual, const T* __restrict__ y, const T* __restrict__ logits,
+gated_norm_add_kernel(float* __restrict__ residual, const T* __restrict__ y, const T* __restrict__ logits, int ldg,
                       const float* __restrict__ bias, const float* __restrict__ gain, float eps, float mult,
                       const float* __restrict__ next_gain, float next_eps, T* __restrict__ out, int d) {
     __shared__ float scratch[16];
-    const size_t base = (size_t)blockIdx.x * d;
+    const size_t base = (size_t)blockIdx.x * d, gbase = (size_t)blockIdx.x * ldg;
     float ss = 0.f;
     for (int c = threadIdx.x; c < d; c += blockDim.x) {
         float g = to_float(y[base + c]);
-        if (logits) g *= soc_sigmoid(to_float(logits[base + c]) + bias[c]);
+        if (logits) g *= soc_sigmoid(to_float(logits[gbase + c]) + bias[c]);
         ss += g * g;
     }
     ss = block_sum(ss, scratch);
@@ -46,7 +47,7 @@ gated_norm_add_kernel(float* __restrict__ residual, const T* __restrict__ y, con
     float rr = 0.f;
     for (int c = threadIdx.x; c < d; c += blockDim.x) {
         float g = to_float(y[base + c]);
-        if (logits) g *= soc_sigmoid(to_float(logits[base + c]) + bias[c]);
+        if (logits) g *= soc_sigmoid(to_float(logits[gbase + c]) + bias[c]);
         const float r = residual[base + c] + scale * gain[c] * g;
         residual[base + c] = r;
         rr += r * r;
@@ -62,18 +63,18 @@ gated_norm_add_kernel(float* __restrict__ residual, const T* __restrict__ y, con
 // read once, all loads are issued before the first is used.
 template <typename T, int PER>
 __global__ void __launch_bounds__(256)
-gated_norm_add_regs_kernel(float* __restrict__ residual, const T* __restrict__ y, const T* __restrict__ logits,
+gated_norm_add_regs_kernel(float* __restrict__ residual, const T* __restrict__ y, const T* __restrict__ logits, int ldg,
                            const float* __restrict__ bias, const float* __restrict__ gain, float eps, float mult,
                            const float* __restrict__ next_gain, float next_eps, T* __restrict__ out, int d) {
     __shared__ float scratch[16];
-    const size_t base = (size_t)blockIdx.x * d;
+    const size_t base = (size_t)blockIdx.x * d, gbase = (size_t)blockIdx.x * ldg;
     float g[PER], res[PER], gate[PER], gn[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
         const int c = threadIdx.x + i * 256;
         const bool in = c < d;
         g[i] = in ? to_float(y[base + c]) : 0.f;
-        gate[i] = (in && logits) ? to_float(logits[base + c]) + bias[c] : 0.f;
+        gate[i] = (in && logits) ? to_float(logits[gbase + c]) + bias[c] : 0.f;
         res[i] = in ? residual[base + c] : 0.f;
         gn[i] = in ? gain[c] : 0.f;
     }
@@ -113,11 +114,11 @@ gated_norm_add_regs_kernel(float* __restrict__ residual, const T* __restrict__ y
 // the first loads, so the kernel waits for memory once.
 template <typename T, int CH>
 __global__ void __launch_bounds__(256)
-gated_norm_add_vec8_kernel(float* __restrict__ residual, const T* __restrict__ y, const T* __restrict__ logits,
+gated_norm_add_vec8_kernel(float* __restrict__ residual, const T* __restrict__ y, const T* __restrict__ logits, int ldg,
                            const float* __restrict__ bias, const float* __restrict__ gain, float eps, float mult,
                            const float* __restrict__ next_gain, float next_eps, T* __restrict__ out, int d) {
     __shared__ float scratch[16];
-    const size_t base = (size_t)blockIdx.x * d;
+    const size_t base = (size_t)blockIdx.x * d, gbase = (size_t)blockIdx.x * ldg;
     float g[CH][8], res[CH][8], gate[CH][8], gn[CH][8], nx[CH][8];
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
@@ -128,7 +129,7 @@ gated_norm_add_vec8_kernel(float* __restrict__ residual, const T* __restrict__ y
             VecLoad<float, 8>::load(gain + c, gn[i]);
             if (logits) {
                 float b[8];
-                VecLoad<T, 8>::load(logits + base + c, gate[i]);
+                VecLoad<T, 8>::load(logits + gbase + c, gate[i]);
                 VecLoad<float, 8>::load(bias + c, b);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) gate[i][e] += b[e];
@@ -173,59 +174,62 @@ gated_norm_add_vec8_kernel(float* __restrict__ residual, const T* __restrict__ y
 }
 
 template <typename T>
-static void launch_gated_norm_add(float* residual, const void* y, const void* logits, const float* bias, const float* gain,
+static void launch_gated_norm_add(float* residual, const void* y, const void* logits, int ldg, const float* bias, const float* gain,
                                   float eps, float mult, const float* next_gain, float next_eps, void* out, int N, int d,
                                   hipStream_t stream) {
 #define SOC_GNA(PER)                                                                                                    \
     hipLaunchKernelGGL((gated_norm_add_regs_kernel<T, PER>), dim3(N), dim3(256), 0, stream, residual, (const T*)y,     \
-                       (const T*)logits, bias, gain, eps, mult, next_gain, next_eps, (T*)out, d)
+                       (const T*)logits, ldg, bias, gain, eps, mult, next_gain, next_eps, (T*)out, d)
 #define SOC_GNA8(CH)                                                                                                    \
     hipLaunchKernelGGL((gated_norm_add_vec8_kernel<T, CH>), dim3(N), dim3(256), 0, stream, residual, (const T*)y,      \
-                       (const T*)logits, bias, gain, eps, mult, next_gain, next_eps, (T*)out, d)
-    if (d % 8 == 0 && d <= 2048) SOC_GNA8(1);
-    else if (d % 8 == 0 && d <= 4096) SOC_GNA8(2);
-    else if (d % 8 == 0 && d <= 8192) SOC_GNA8(4);
+                       (const T*)logits, ldg, bias, gain, eps, mult, next_gain, next_eps, (T*)out, d)
+    // (pieces of eight elements: the width, the logits' rows and their first element all sit at multiples of 8)
+    const bool by8 = d % 8 == 0 && ldg % 8 == 0 && ((uintptr_t)logits % (8 * sizeof(T))) == 0;
+    if (by8 && d <= 2048) SOC_GNA8(1);
+    else if (by8 && d <= 4096) SOC_GNA8(2);
+    else if (by8 && d <= 8192) SOC_GNA8(4);
     else if (d <= 1024) SOC_GNA(4);
     else if (d <= 2048) SOC_GNA(8);
     else if (d <= 4096) SOC_GNA(16);
     else if (d <= 8192) SOC_GNA(32);
     else
         hipLaunchKernelGGL(gated_norm_add_kernel<T>, dim3(N), dim3(256), 0, stream, residual, (const T*)y, (const T*)logits,
-                           bias, gain, eps, mult, next_gain, next_eps, (T*)out, d);
+                           ldg, bias, gain, eps, mult, next_gain, next_eps, (T*)out, d);
 }
 
-SOC_EXPORT int soc_gated_norm_add(float* residual, const void* y, const void* logits, const float* bias,
+SOC_EXPORT int soc_gated_norm_add(float* residual, const void* y, const void* logits, int ldg, const float* bias,
                                   const float* gain, float eps, float mult, const float* next_gain, float next_eps,
                                   void* out, int N, int d, int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
-    if (dtype == 0) launch_gated_norm_add<float>(residual, y, logits, bias, gain, eps, mult, next_gain, next_eps, out, N, d, stream);
-    else launch_gated_norm_add<bf16>(residual, y, logits, bias, gain, eps, mult, next_gain, next_eps, out, N, d, stream);
+    if (dtype == 0) launch_gated_norm_add<float>(residual, y, logits, ldg, bias, gain, eps, mult, next_gain, next_eps, out, N, d, stream);
+    else launch_gated_norm_add<bf16>(residual, y, logits, ldg, bias, gain, eps, mult, next_gain, next_eps, out, N, d, stream);
     return soc_last_error();
 }
 
 // ---- g * sigmoid(slope g) * (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit) ---------
+// gate and up are the first 2 ff elements of rows of ld elements.
 template <typename T>
-__global__ void glu_clamped_kernel(const T* __restrict__ gate_up, T* __restrict__ out, size_t total, int ff,
+__global__ void glu_clamped_kernel(const T* __restrict__ gate_up, T* __restrict__ out, size_t total, int ff, int ld,
                                    float limit, float slope) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
     const size_t n = i / ff, c = i % ff;
-    const float g = fminf(to_float(gate_up[n * 2 * ff + c]), limit);
-    const float u = fminf(fmaxf(to_float(gate_up[n * 2 * ff + ff + c]), -limit), limit);
+    const float g = fminf(to_float(gate_up[n * ld + c]), limit);
+    const float u = fminf(fmaxf(to_float(gate_up[n * ld + ff + c]), -limit), limit);
     out[i] = from_float<T>(g * soc_sigmoid(slope * g) * (u + 1.f));
 }
 
 // (eight consecutive elements per lane where ff is a multiple of 8)
 template <typename T>
-__global__ void glu_clamped_vec8_kernel(const T* __restrict__ gate_up, T* __restrict__ out, size_t groups, int ff,
+__global__ void glu_clamped_vec8_kernel(const T* __restrict__ gate_up, T* __restrict__ out, size_t groups, int ff, int ld,
                                         float limit, float slope) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= groups) return;
     const int per_row = ff / 8;
     const size_t n = i / per_row, c = (i % per_row) * 8;
     float g[8], u[8], y[8];
-    VecLoad<T, 8>::load(gate_up + n * 2 * ff + c, g);
-    VecLoad<T, 8>::load(gate_up + n * 2 * ff + ff + c, u);
+    VecLoad<T, 8>::load(gate_up + n * ld + c, g);
+    VecLoad<T, 8>::load(gate_up + n * ld + ff + c, u);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         const float gg = fminf(g[e], limit), uu = fminf(fmaxf(u[e], -limit), limit);
@@ -234,28 +238,29 @@ __global__ void glu_clamped_vec8_kernel(const T* __restrict__ gate_up, T* __rest
     store8(out + n * ff + c, y);
 }
 
-SOC_EXPORT int soc_glu_clamped(const void* gate_up, void* out, int N, int ff, float limit, float slope, int dtype,
+SOC_EXPORT int soc_glu_clamped(const void* gate_up, void* out, int N, int ff, int ld, float limit, float slope, int dtype,
                                hipStream_t stream) {
     const size_t total = (size_t)N * ff;
     if (total == 0) return 0;
-    if (ff % 8 == 0) {
+    if (ld < 2 * ff) return (int)hipErrorInvalidValue;
+    if (ff % 8 == 0 && ld % 8 == 0) {
         const size_t groups = total / 8;
         const dim3 grid((unsigned)((groups + 255) / 256));
         if (dtype == 0)
             hipLaunchKernelGGL(glu_clamped_vec8_kernel<float>, grid, dim3(256), 0, stream, (const float*)gate_up, (float*)out,
-                               groups, ff, limit, slope);
+                               groups, ff, ld, limit, slope);
         else
             hipLaunchKernelGGL(glu_clamped_vec8_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)gate_up, (bf16*)out,
-                               groups, ff, limit, slope);
+                               groups, ff, ld, limit, slope);
         return soc_last_error();
     }
     const dim3 grid((unsigned)((total + 255) / 256));
     if (dtype == 0)
         hipLaunchKernelGGL(glu_clamped_kernel<float>, grid, dim3(256), 0, stream, (const float*)gate_up, (float*)out,
-                           total, ff, limit, slope);
+                           total, ff, ld, limit, slope);
     else
         hipLaunchKernelGGL(glu_clamped_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)gate_up, (bf16*)out,
-                           total, ff, limit, slope);
+                           total, ff, ld, limit, slope);
     return soc_last_error();
 }
 

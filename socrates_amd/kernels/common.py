@@ -52,8 +52,8 @@ _GEMM_SIGNATURES = {
 }
 L = c_longlong
 _MIXER_SIGNATURES = {
-    "soc_gated_norm_add": [P, P, P, P, P, F, F, P, F, P, I, I, I, P],
-    "soc_glu_clamped": [P, P, I, I, F, F, I, P],
+    "soc_gated_norm_add": [P, P, P, I, P, P, F, F, P, F, P, I, I, I, P],
+    "soc_glu_clamped": [P, P, I, I, I, F, F, I, P],
     "soc_token_shift": [P, P, I, P, L, I, P, P, P, I, I, I, I, I, P],
     "soc_wkv_decay": [P, P, P, P, I, I, I, I, P],
     "soc_wkv": [P, P, P, P, P, I, I, P, L, I, P, P, P, I, I, I, P],

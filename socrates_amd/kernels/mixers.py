@@ -24,32 +24,42 @@ class Mixers:
     def gated_norm_add(self, residual, y, gate_logits, gate_bias, gain, eps, mult, next_gain=None, next_eps=0.0):
         """residual (float32 [N, d], in place) += mult * gain * g / rms(g) with g = y *
         sigmoid(gate_logits + gate_bias) (no gate: g = y). With ``next_gain``: returns
-        residual / rms(residual) * next_gain in the compute dtype; else None."""
+        residual / rms(residual) * next_gain in the compute dtype; else None. ``gate_logits`` may be
+        [N, d] columns of a wider product (rows apart by its width)."""
         N, d = residual.shape
         self._want(residual, "residual", torch.float32)
         self._want(y, "branch result", self.dtype, (N, d))
         self._want(gain, "norm gain", torch.float32, (d,))
+        ldg = 0
         if gate_logits is not None:
-            self._want(gate_logits, "gate", self.dtype, (N, d))
+            if (gate_logits.device.type != "cuda" or gate_logits.dtype != self.dtype or tuple(gate_logits.shape) != (N, d)
+                    or gate_logits.stride(1) != 1 or gate_logits.stride(0) < d):
+                raise KernelError(f"gate logits {tuple(gate_logits.shape)} with strides {gate_logits.stride()} do not fit [{N}, {d}]")
+            ldg = gate_logits.stride(0)
             self._want(gate_bias, "gate bias", torch.float32, (d,))
         out = None
         if next_gain is not None:
             self._want(next_gain, "next norm's gain", torch.float32, (d,))
             out = torch.empty((N, d), dtype=self.dtype, device=self.device)
         _check(self._mixers().soc_gated_norm_add(
-            _ptr(residual), _ptr(y), _ptr(gate_logits), _ptr(gate_bias if gate_logits is not None else None), _ptr(gain),
+            _ptr(residual), _ptr(y), _ptr(gate_logits), c_int(ldg), _ptr(gate_bias if gate_logits is not None else None), _ptr(gain),
             c_float(eps), c_float(mult), _ptr(next_gain), c_float(next_eps), _ptr(out), c_int(N), c_int(d),
             c_int(self.code), self._stream()), "gated_norm_add")
         return out
 
-    def glu_clamped(self, gate_up, limit, slope):
-        """[N, gate | up] -> g * sigmoid(slope g) * (u + 1), g = min(gate, limit), u = clamp(up, +-limit)."""
+    def glu_clamped(self, gate_up, limit, slope, ff=None):
+        """[N, gate | up] -> g * sigmoid(slope g) * (u + 1), g = min(gate, limit), u = clamp(up, +-limit).
+        With ``ff``: gate and up are the first 2 ff columns of a wider product."""
         self._want(gate_up, "gate and up", self.dtype)
-        N, two_ff = gate_up.shape
-        if two_ff % 2:
-            raise KernelError("gate and up have the same number of columns")
-        out = torch.empty((N, two_ff // 2), dtype=self.dtype, device=self.device)
-        _check(self._mixers().soc_glu_clamped(_ptr(gate_up), _ptr(out), c_int(N), c_int(two_ff // 2), c_float(limit),
+        N, ld = gate_up.shape
+        if ff is None:
+            if ld % 2:
+                raise KernelError("gate and up have the same number of columns")
+            ff = ld // 2
+        if ff < 1 or 2 * ff > ld:
+            raise KernelError(f"{ld} columns do not hold gate and up of {ff}")
+        out = torch.empty((N, ff), dtype=self.dtype, device=self.device)
+        _check(self._mixers().soc_glu_clamped(_ptr(gate_up), _ptr(out), c_int(N), c_int(ff), c_int(ld), c_float(limit),
                                               c_float(slope), c_int(self.code), self._stream()), "glu_clamped")
         return out
 

@@ -132,6 +132,11 @@ class SandwichBlock:
             setattr(self, role, None if sub is None else build_part(sub, _sub_tensors(spec, role, weights), ops))
         if self.ffn is not None and (self.norm2 is None or self.post_norm2 is None):
             raise ValueError("a feed-forward needs the norms before and after it")
+        # A branch whose first product reads its input as it comes takes the gate's matrix as further rows of
+        # that product (``adopt``): one launch less, and the gate's logits come back beside the branch's result.
+        for part, gate in ((self.mixer, self.gate1), (self.ffn, self.gate2)):
+            if gate is not None and hasattr(part, "adopt"):
+                gate.weight = part.adopt(gate.weight)
         parts = [getattr(self, role) for role in spec.ROLES]
         self.capturable = all(getattr(p, "capturable", True) for p in parts if p is not None)
 
@@ -142,11 +147,14 @@ class SandwichBlock:
                 part.reserve(n_positions)
 
     def _close(self, residual, y, h, gate, post_norm, next_norm):
-        """Close a branch whose input was ``h`` and whose result is ``y``; returns the rows
-        the next branch reads (None if nothing follows in this stream)."""
+        """Close a branch whose input was ``h`` and whose result is ``y`` (or (result, gate logits) from a
+        branch that has adopted the gate's matrix); returns the rows the next branch reads (None if nothing
+        follows in this stream)."""
         ops = self.ops
         logits = bias = None
-        if gate is not None:
+        if isinstance(y, tuple):
+            (y, logits), bias = y, gate.bias
+        elif gate is not None:
             logits, bias = ops.linear(h, gate.weight), gate.bias
         gain, eps = post_norm.fusable()
         follows = next_norm.fusable() if hasattr(next_norm, "fusable") else None

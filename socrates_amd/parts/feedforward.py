@@ -58,10 +58,21 @@ class ClampedGLU:
         # one operand for gate and up: rows [gate | up]
         self.w_gate_up = torch.cat([tensors["gate"], tensors["up"]], dim=0).contiguous()
         self.w_down = tensors["down"]
+        self.adopted = 0
+
+    def adopt(self, w):
+        """Take ``w`` [n, hidden] as further rows of the first product; ``forward`` then returns (y, x w^T).
+        Returns the rows as they now lie (a view), for whoever held ``w``."""
+        self.w_gate_up = torch.cat([self.w_gate_up, w], dim=0).contiguous()
+        self.adopted = w.shape[0]
+        return self.w_gate_up[2 * self.spec.intermediate:]
 
     def forward(self, x, ctx=None):
-        act = self.ops.glu_clamped(self.ops.linear(x, self.w_gate_up), self.spec.limit, self.spec.slope)
-        return self.ops.linear(act, self.w_down)
+        ff = self.spec.intermediate
+        both = self.ops.linear(x, self.w_gate_up)
+        act = self.ops.glu_clamped(both, self.spec.limit, self.spec.slope, ff)
+        y = self.ops.linear(act, self.w_down)
+        return (y, both[:, 2 * ff:]) if self.adopted else y
 
 
 class SigmoidGate:

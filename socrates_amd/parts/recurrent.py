@@ -79,16 +79,25 @@ class Mamba2Mixer:
         self.conv, self.conv_bias = tensors["conv"], tensors["conv.b"]
         self.dt_bias, self.a_log, self.skip = tensors["dt_bias"], tensors["A_log"], tensors["D"]
         self.gain, self.w_o = tensors["norm"], tensors["o"]
+        self.adopted = 0
+
+    def adopt(self, w):
+        """Take ``w`` [n, hidden] as further rows of the input projection; ``forward`` then returns
+        (y, x w^T). Returns the rows as they now lie (a view), for whoever held ``w``."""
+        n = self.w_main.shape[0]
+        self.w_main = torch.cat([self.w_main, w], dim=0).contiguous()
+        self.adopted = w.shape[0]
+        return self.w_main[n:]
 
     def forward(self, x, ctx, slot, write=True):
         s, ops = self.spec, self.ops
-        zxbc = ops.linear(x, self.w_main)                                  # [N, z | x B C]
+        zxbc = ops.linear(x, self.w_main)                                  # [N, z | x B C (| what was adopted)]
         dt = ops.linear(x, self.w_dt, out_dtype=torch.float32)
         xbc = ops.causal_conv_silu(zxbc, s.inner, s.conv_channels, self.conv, self.conv_bias, slot.state, 0, ctx)
         y = ops.ssd(xbc, dt, self.dt_bias, self.a_log, self.skip, s.n_heads, s.head_dim, s.state, s.n_groups,
                     slot.state, (s.conv_taps - 1) * s.conv_channels, ctx)
-        y = ops.gated_group_norm(y, zxbc, self.gain, s.norm_groups, s.eps)
-        return ops.linear(y, self.w_o)
+        y = ops.linear(ops.gated_group_norm(y, zxbc, self.gain, s.norm_groups, s.eps), self.w_o)
+        return (y, zxbc[:, s.inner + s.conv_channels:]) if self.adopted else y
 
 
 register_part(WkvSpec, WkvMixer)

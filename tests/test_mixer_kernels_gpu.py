@@ -61,6 +61,16 @@ def test_gated_norm_add(kernel_sets, dtype, N, d, gated, follows):
     assert (a is None) == (not follows)
     if follows:
         close(a, b, dtype)
+    if gated:
+        # the logits as columns of a wider product, at an offset that is a multiple of 8 and at one that is not
+        for off in (16, 3):
+            wide = rnd((N, off + d + 5), dtype, 7)
+            wide[:, off:off + d] = logits
+            r3 = res.clone()
+            a3 = hip.gated_norm_add(r3, y, wide[:, off:off + d], bias, gain, 1e-5, 0.7, nxt, 1e-6)
+            torch.testing.assert_close(r3, r1, atol=1e-6, rtol=1e-6)
+            if follows:
+                close(a3, a, dtype, atol=1e-6 if dtype == torch.float32 else 1e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -69,6 +79,9 @@ def test_glu_clamped(kernel_sets, dtype):
     for ff in (93, 96, 1000):
         x = rnd((7, 2 * ff), dtype, 1, 2.0)
         close(hip.glu_clamped(x, 1.5, 1.702), ref.glu_clamped(x, 1.5, 1.702), dtype)
+        for extra in (8, 13):           # gate and up as the first columns of a wider product
+            wide = torch.cat([x, rnd((7, extra), dtype, 2)], dim=1).contiguous()
+            close(hip.glu_clamped(wide, 1.5, 1.702, ff), ref.glu_clamped(x, 1.5, 1.702), dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

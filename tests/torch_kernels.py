@@ -170,10 +170,10 @@ class TorchKernels:
             return None
         return self._norm(residual, next_gain, next_eps).to(self.dtype)
 
-    def glu_clamped(self, gate_up, limit, slope):
-        ff = gate_up.shape[-1] // 2
+    def glu_clamped(self, gate_up, limit, slope, ff=None):
+        ff = ff or gate_up.shape[-1] // 2
         g = torch.clamp(gate_up[..., :ff].to(self.acc), max=limit)
-        u = torch.clamp(gate_up[..., ff:].to(self.acc), min=-limit, max=limit)
+        u = torch.clamp(gate_up[..., ff:2 * ff].to(self.acc), min=-limit, max=limit)
         return (g * torch.sigmoid(slope * g) * (u + 1)).to(self.dtype)
 
     # -- mixers with a state per row -------------------------------------------------------------
