@@ -81,6 +81,29 @@ def test_drawn_configurations(tmp_path, kernel_sets, seed, dtype):
 
 
 @pytest.mark.parametrize("dtype", list(DTYPES))
+def test_a_wider_model_with_long_prompts(tmp_path, kernel_sets, dtype):
+    """Width 320, six layers, heads of 48 and 96, states of 64 and 128, a latent of 96 + 24 (padded to 128 in its
+    pages), windows of 100 and 37 on one cache, prompts of up to 700 tokens: decoded at the end, mixed, and in
+    portions of 2 to 200 tokens, through captured decode steps."""
+    from helpers import trace_mixed, trace_portions
+    cfg = model(320, 500, [latent(5, 48, 24, 40, 96, 64, window=100, scale=0.15), wkv(5, 48),
+                           mamba2(6, 40, 64, groups=2, conv=3, norm_groups=2),
+                           latent(7, 32, 24, 56, 96, 72, window=37, scale=0.2, kv_from=0), wkv(4, 96),
+                           mamba2(4, 64, 128, groups=1, conv=4, norm_groups=1)], ff=520, limit=2.0, mult=0.7, no_ff=(4,))
+    folder = write_model(tmp_path / "m", cfg, seed=5)
+    prompts = random_prompts([700, 333, 64, 150], cfg["vocab"], seed=6)
+    want = oracle(folder, prompts)
+    tol = TOL[dtype] if dtype == "float32" else (0.2, 0.06)
+    for name, steps in (("tail", trace_tail_decode(prompts, 40)), ("mixed", trace_mixed(prompts, seed=7)),
+                        ("portions", trace_portions(prompts, seed=8, sizes=(2, 3, 64, 65, 128, 200)))):
+        runner = make_runner(folder, kernel_sets[dtype], max_rows=4, max_len=768, block_size=16, num_blocks=4 * 48)
+        runner.enable_graphs(4)
+        got = replay(runner, steps)
+        for i in range(len(prompts)):
+            compare(got[f"r{i}"], want[i], tol, f"{name} {dtype} request {i}")
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
 @pytest.mark.parametrize("heads", [17, 20, 33])
 def test_many_heads_on_one_cached_vector(tmp_path, kernel_sets, heads, dtype):
     """All heads of a latent-attention layer share one cached vector, one "kv head" for the attention kernels:
