@@ -715,18 +715,46 @@ SOC_EXPORT int soc_gated_group_norm(const float* y, const void* z, int ldz, cons
     return soc_last_error();
 }
 
+// ---- RMS norm of the first dim elements of rows of ld elements, into rows of dim -------------------------------
+// (a query latent that is some of the columns of a wider product). One wave per row.
+template <typename T>
+__global__ void __launch_bounds__(256)
+rmsnorm_cols_kernel(const T* __restrict__ x, int ld, const float* __restrict__ w, T* __restrict__ out, int N, int dim,
+                    float eps) {
+    const int n = blockIdx.x * (256 / SOC_WAVE) + threadIdx.x / SOC_WAVE, lane = threadIdx.x % SOC_WAVE;
+    if (n >= N) return;
+    const T* row = x + (size_t)n * ld;
+    float ss = 0.f;
+    for (int c = lane; c < dim; c += SOC_WAVE) { const float v = to_float(row[c]); ss += v * v; }
+    ss = wave_sum(ss);
+    const float inv = 1.f / sqrtf(ss / (float)dim + eps);
+    for (int c = lane; c < dim; c += SOC_WAVE) out[(size_t)n * dim + c] = from_float<T>(to_float(row[c]) * inv * w[c]);
+}
+
+SOC_EXPORT int soc_rmsnorm_cols(const void* x, int ld, const float* w, void* out, int N, int dim, float eps, int dtype,
+                                hipStream_t stream) {
+    if (N <= 0) return 0;
+    if (dim < 1 || ld < dim) return (int)hipErrorInvalidValue;
+    const dim3 grid((N + 3) / 4);
+    if (dtype == 0)
+        hipLaunchKernelGGL(rmsnorm_cols_kernel<float>, grid, dim3(256), 0, stream, (const float*)x, ld, w, (float*)out, N, dim, eps);
+    else
+        hipLaunchKernelGGL(rmsnorm_cols_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)x, ld, w, (bf16*)out, N, dim, eps);
+    return soc_last_error();
+}
+
 // ---- a token's latent into its page ---------------------------------------------------------------------------
-// kvd [N, R + Dr]: the first R RMS-normed with gain, the rest turned pair by pair (pairs 2i, 2i + 1 of the
+// kvd: the first R + Dr elements of rows of ld elements: the first R RMS-normed with gain, the rest turned pair by pair (pairs 2i, 2i + 1 of the
 // first 2 * half by position * inv_freq[i]); both go to the token's place in the pool
 // [pages, 1, block, width], the padding up to width as zeros. One wave per token.
 template <typename T>
 __global__ void __launch_bounds__(64)
-latent_write_kernel(const T* __restrict__ kvd, int R, int Dr, const float* __restrict__ gain, float eps,
+latent_write_kernel(const T* __restrict__ kvd, int ld, int R, int Dr, const float* __restrict__ gain, float eps,
                     const float* __restrict__ inv_freq, int half, const int* __restrict__ positions,
                     const int* __restrict__ token_rows, const int* __restrict__ table, int table_width,
                     T* __restrict__ pool, int block, int width) {
     const int n = blockIdx.x, lane = threadIdx.x;
-    const T* row = kvd + (size_t)n * (R + Dr);
+    const T* row = kvd + (size_t)n * ld;
     const int pos = positions[n];
     const int page = table[(size_t)token_rows[n] * table_width + pos / block];
     T* dst = pool + ((size_t)page * block + pos % block) * width;
@@ -751,16 +779,16 @@ latent_write_kernel(const T* __restrict__ kvd, int R, int Dr, const float* __res
     for (int c = R + Dr + lane; c < width; c += 64) dst[c] = from_float<T>(0.f);
 }
 
-SOC_EXPORT int soc_latent_write(const void* kvd, int N, int R, int Dr, const float* gain, float eps, const float* inv_freq,
+SOC_EXPORT int soc_latent_write(const void* kvd, int ld, int N, int R, int Dr, const float* gain, float eps, const float* inv_freq,
                                 int half, const int* positions, const int* token_rows, const int* table, int table_width,
                                 void* pool, int block, int width, int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
-    if (2 * half > Dr || R + Dr > width) return (int)hipErrorInvalidValue;
+    if (2 * half > Dr || R + Dr > width || ld < R + Dr) return (int)hipErrorInvalidValue;
     if (dtype == 0)
-        hipLaunchKernelGGL(latent_write_kernel<float>, dim3(N), dim3(64), 0, stream, (const float*)kvd, R, Dr, gain, eps, inv_freq,
+        hipLaunchKernelGGL(latent_write_kernel<float>, dim3(N), dim3(64), 0, stream, (const float*)kvd, ld, R, Dr, gain, eps, inv_freq,
                            half, positions, token_rows, table, table_width, (float*)pool, block, width);
     else
-        hipLaunchKernelGGL(latent_write_kernel<bf16>, dim3(N), dim3(64), 0, stream, (const bf16*)kvd, R, Dr, gain, eps, inv_freq,
+        hipLaunchKernelGGL(latent_write_kernel<bf16>, dim3(N), dim3(64), 0, stream, (const bf16*)kvd, ld, R, Dr, gain, eps, inv_freq,
                            half, positions, token_rows, table, table_width, (bf16*)pool, block, width);
     return soc_last_error();
 }

@@ -60,7 +60,8 @@ _MIXER_SIGNATURES = {
     "soc_causal_conv_silu": [P, I, I, I, P, P, I, P, L, I, P, P, P, I, I, I, P],
     "soc_ssd": [P, P, P, P, P, I, I, I, I, P, L, I, P, P, P, I, I, I, P],
     "soc_gated_group_norm": [P, P, I, P, I, I, I, F, I, P, I, P],
-    "soc_latent_write": [P, I, I, I, P, F, P, I, P, P, P, I, P, I, I, I, P],
+    "soc_latent_write": [P, I, I, I, I, P, F, P, I, P, P, P, I, P, I, I, I, P],
+    "soc_rmsnorm_cols": [P, I, P, P, I, I, F, I, P],
     "soc_latent_query_turn": [P, I, I, I, I, I, I, P, I, P, P, I, P],
     "soc_head_linear": [P, I, P, P, I, I, I, I, I, I, P],
 }

@@ -176,11 +176,28 @@ class Mixers:
         return out
 
     # -- attention over a cached latent ---------------------------------------------------------------------
+    def _columns(self, x, name, N, dim):
+        """``x`` is [N, dim] in the compute dtype, rows contiguous and apart by at least ``dim`` (columns of a
+        wider product)."""
+        if (x.device.type != "cuda" or x.dtype != self.dtype or tuple(x.shape) != (N, dim) or x.stride(1) != 1
+                or x.stride(0) < dim):
+            raise KernelError(f"{name}: {tuple(x.shape)} with strides {x.stride()} does not fit [{N}, {dim}]")
+
+    def rmsnorm_cols(self, x, weight, eps):
+        """RMS norm of ``x`` [N, dim], which may be columns of a wider product; returns contiguous rows."""
+        N, dim = x.shape
+        self._columns(x, "x", N, dim)
+        self._want(weight, "norm weight", torch.float32, (dim,))
+        out = torch.empty((N, dim), dtype=self.dtype, device=self.device)
+        _check(self._mixers().soc_rmsnorm_cols(_ptr(x), c_int(x.stride(0)), _ptr(weight), _ptr(out), c_int(N), c_int(dim),
+                                               c_float(eps), c_int(self.code), self._stream()), "rmsnorm_cols")
+        return out
+
     def latent_write(self, kvd, R, Dr, gain, eps, inv_freq, positions, token_rows, slot):
-        """kvd [N, R + Dr]: the first R RMS-normed, the rest turned by position, into each token's place
-        of the pool [pages, 1, block, width]."""
+        """kvd [N, R + Dr] (it may be columns of a wider product): the first R RMS-normed, the rest turned by
+        position, into each token's place of the pool [pages, 1, block, width]."""
         N = kvd.shape[0]
-        self._want(kvd, "latent and key part", self.dtype, (N, R + Dr))
+        self._columns(kvd, "latent and key part", N, R + Dr)
         self._want(gain, "latent gain", torch.float32, (R,))
         self._want(inv_freq, "inv_freq", torch.float32)
         self._want(positions, "positions", torch.int32, (N,))
@@ -192,7 +209,8 @@ class Mixers:
                 or 2 * inv_freq.numel() > Dr:
             raise KernelError(f"latent pool {tuple(slot.k.shape)} does not fit {R} + {Dr} elements per token")
         _check(self._mixers().soc_latent_write(
-            _ptr(kvd), c_int(N), c_int(R), c_int(Dr), _ptr(gain), c_float(eps), _ptr(inv_freq), c_int(inv_freq.numel()),
+            _ptr(kvd), c_int(kvd.stride(0)), c_int(N), c_int(R), c_int(Dr), _ptr(gain), c_float(eps), _ptr(inv_freq),
+            c_int(inv_freq.numel()),
             _ptr(positions), _ptr(token_rows), _ptr(slot.block_table), c_int(slot.block_table.shape[1]), _ptr(slot.k),
             c_int(slot.block_size), c_int(width), c_int(self.code), self._stream()), "latent_write")
 

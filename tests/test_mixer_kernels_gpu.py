@@ -213,6 +213,13 @@ def test_latent_write_and_query(kernel_sets, dtype, R, Dr, dims, width, block):
     hip.latent_write(kvd, R, Dr, gain, 1e-5, inv_freq, positions, rows, s1)
     ref.latent_write(kvd, R, Dr, gain, 1e-5, inv_freq, positions, rows, s2)
     close(s1.k, s2.k, dtype)
+    # the same rows as columns of a wider product
+    wide = rnd((N, 7 + R + Dr + 3), dtype, 9)
+    wide[:, 7:7 + R + Dr] = kvd
+    s3 = SimpleNamespace(k=torch.zeros_like(s1.k), v=None, block_table=s1.block_table, block_size=block, window=None)
+    hip.latent_write(wide[:, 7:7 + R + Dr], R, Dr, gain, 1e-5, inv_freq, positions, rows, s3)
+    torch.testing.assert_close(s3.k, s1.k, atol=0, rtol=0)
+    close(hip.rmsnorm_cols(wide[:, 7:7 + R], gain, 1e-5), ref.rmsnorm_cols(kvd[:, :R], gain, 1e-5), dtype)
     q, w = rnd((N, H * (D + Dr)), dtype, 3), rnd((H, R, D), dtype, 4, 0.3)
     close(hip.latent_query(q, H, D, Dr, w, width, inv_freq, positions), ref.latent_query(q, H, D, Dr, w, width, inv_freq, positions),
           dtype, atol=5e-5 if dtype == torch.float32 else 3e-2)

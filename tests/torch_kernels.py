@@ -271,6 +271,9 @@ class TorchKernels:
         out[..., 1:dims:2] = b * cos + a * sin
         return out
 
+    def rmsnorm_cols(self, x, weight, eps):
+        return self._norm(x, weight, eps).to(self.dtype)
+
     def latent_write(self, kvd, R, Dr, gain, eps, inv_freq, positions, token_rows, slot):
         A = self.acc
         latent = self._norm(kvd[:, :R], gain, eps)
