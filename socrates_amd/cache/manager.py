@@ -58,6 +58,10 @@ class PagedGroup:
         # per row: number of logical blocks ever covered, and the first one still held
         self.covered = [0] * max_rows
         self.first_live = [0] * max_rows
+        # with a window that keeps the first positions visible: the blocks that hold them stay with the
+        # row whatever the window has passed (a row then holds blocks 0 .. kept and first_live .. covered)
+        keep_first = getattr(need, "keep_first", 0) if need.window is not None else 0
+        self.kept_blocks = blocks_for(keep_first, block_size) if keep_first > 0 else 0
         self.dirty = set()
         # a latent is kept as one "head" of ``width`` elements, in one pool per slot
         self.pool_shape = ((num_blocks + 1, 1, block_size, need.width) if isinstance(need, PagedLatent)
@@ -80,12 +84,25 @@ class PagedGroup:
         first_visible = max(0, next_start - self.need.window + 1)
         return max(self.first_live[row], min(first_visible // self.block_size, self.covered[row]))
 
+    def _held(self, row: int):
+        """The logical blocks ``row`` holds: the kept first ones and those from first_live on."""
+        a = min(self.kept_blocks, self.covered[row])
+        b = max(self.first_live[row], a)
+        return list(range(a)) + list(range(b, self.covered[row]))
+
+    def would_free(self, row: int, next_start: int) -> int:
+        """How many pages ``drop_behind`` would give back."""
+        return max(0, self.droppable(row, next_start) - max(self.first_live[row], min(self.kept_blocks, self.covered[row])))
+
+    def held_count(self, row: int) -> int:
+        return len(self._held(row))
+
     def missing(self, row: int, new_len: int) -> int:
         return max(0, blocks_for(new_len, self.block_size) - self.covered[row])
 
     def drop_behind(self, row: int, next_start: int):
         upto = self.droppable(row, next_start)
-        lo = self.first_live[row]
+        lo = max(self.first_live[row], min(self.kept_blocks, self.covered[row]))
         if upto > lo:
             pages = [int(p) for p in self.host_table[row, lo:upto]]
             self.allocator.free(pages)
@@ -104,16 +121,17 @@ class PagedGroup:
             self.dirty.add(row)
 
     def release(self, row: int):
-        lo, hi = self.first_live[row], self.covered[row]
-        if hi > lo:
-            self.allocator.free([int(p) for p in self.host_table[row, lo:hi]])
+        hi = self.covered[row]
+        held = self._held(row)
+        if held:
+            self.allocator.free([int(p) for p in self.host_table[row, held]])
         if hi:
             self.host_table[row, :hi] = NULL_PAGE
             self.dirty.add(row)
         self.covered[row] = self.first_live[row] = 0
 
     def held_by(self, row: int):
-        return [int(p) for p in self.host_table[row, self.first_live[row]:self.covered[row]]]
+        return [int(p) for p in self.host_table[row, self._held(row)]]
 
     def sync(self):
         if self.dirty:
@@ -164,6 +182,8 @@ class CacheManager:
         by_need = {}
         for slot_id, need in enumerate(needs):
             if isinstance(need, (PagedKV, PagedLatent)):
+                if getattr(need, "keep_first", 0) < 0:
+                    raise ValueError(f"cache slot {slot_id}: keep_first is not negative")
                 group = by_need.get(need)
                 if group is None:
                     group = PagedGroup(need, max_rows, self.table_width, block_size, num_blocks,
@@ -250,8 +270,7 @@ class CacheManager:
         start = self.length(row)
         short = 0
         for g in self.groups:
-            freed = g.droppable(row, start) - g.first_live[row]
-            short = max(short, g.missing(row, new_len) - freed - g.allocator.n_free)
+            short = max(short, g.missing(row, new_len) - g.would_free(row, start) - g.allocator.n_free)
         return max(short, 0)
 
     def pages_needed(self, row: int, new_len: int):
@@ -259,8 +278,7 @@ class CacheManager:
         that step would give back first (may be negative)."""
         self._check_open(row)
         start = self.length(row)
-        return [g.missing(row, new_len) - (g.droppable(row, start) - g.first_live[row])
-                for g in self.groups]
+        return [g.missing(row, new_len) - g.would_free(row, start) for g in self.groups]
 
     def free_pages(self):
         """Per group: pages free now."""
@@ -268,7 +286,7 @@ class CacheManager:
 
     def held_pages(self, row: int):
         """Per group: pages ``row`` holds now."""
-        return [g.covered[row] - g.first_live[row] for g in self.groups]
+        return [g.held_count(row) for g in self.groups]
 
     @property
     def pool_tokens(self) -> int:
@@ -323,9 +341,9 @@ class CacheManager:
                 held = g.held_by(row)
                 if not self._open[row] and (held or g.host_table[row].any()):
                     raise AssertionError(f"group {gi}: closed row {row} holds pages")
-                outside = np.concatenate([g.host_table[row, :g.first_live[row]],
-                                          g.host_table[row, g.covered[row]:]])
-                if outside.any():
+                live = np.zeros(g.table_width, dtype=bool)
+                live[g._held(row)] = True
+                if g.host_table[row, ~live].any():
                     raise AssertionError(f"group {gi}: row {row} has table entries outside its live range")
                 for p in held:
                     if p == NULL_PAGE:

@@ -13,6 +13,7 @@ from pathlib import Path
 
 from .mitisun import MitisunConfig
 from .qwen3 import ConfigError, Qwen3Config
+from .tedulorn import TedulornConfig
 
 _ARCHITECTURES = {}
 
@@ -98,3 +99,4 @@ def load_preset(name: str):
 
 register_architecture("Qwen3ForCausalLM", Qwen3Config)
 register_architecture("Mitisun", MitisunConfig)
+register_architecture("Tedulorn", TedulornConfig)

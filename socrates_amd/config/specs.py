@@ -15,9 +15,11 @@ from typing import Optional, Tuple
 
 @dataclass(frozen=True)
 class RMSNormSpec:
-    """y = x / sqrt(mean(x^2) + eps) * w  over the last ``dim`` elements."""
+    """y = x / sqrt(mean(x^2) + eps) * w  over the last ``dim`` elements. ``tensor``: the local
+    name of w on disk ("": the tensor carries the norm's own name)."""
     dim: int
     eps: float
+    tensor: str = "weight"
 
 
 @dataclass(frozen=True)
@@ -225,6 +227,125 @@ class LatentAttentionSpec:
 
 
 @dataclass(frozen=True)
+class GatedWindowAttentionSpec:
+    """Grouped-query softmax attention whose keys and values may differ in size, over a window that
+    keeps the first tokens visible, with a gate per head.
+
+    q, k [heads x ``head_dim``], v [kv heads x ``v_dim``]; q and k RMS-normed per head with one gain
+    each (``qk_norm_eps`` None: no norm), then turned by ``position``. A query at position p sees key
+    j <= p if p - j < ``window`` or j < ``keep_first`` (``window`` None: all). ``sink`` adds one weight of
+    score 0 and no value to the softmax's sum: p_j = exp(s_j) / (1 + sum exp(s_j)). ``value_blend``
+    "first": the layer's values are what later layers blend with; "later": its values become
+    (1 - l) v + l v_first, with l the stored number ``vmix`` and v_first the "first" layer's values of
+    the same token (the blend is what the cache holds); None: no blend. ``head_gate``: head h's result
+    is multiplied by sigmoid(W_g x)_h before the output projection."""
+    hidden: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    v_dim: int
+    scale: float
+    qk_norm_eps: Optional[float] = None
+    position: Optional[object] = None
+    window: Optional[int] = None
+    keep_first: int = 0
+    sink: bool = False
+    value_blend: Optional[str] = None
+    stores_blend: bool = False           # the file holds ``vmix`` also where the layer does not use it
+    head_gate: bool = False
+
+    def __post_init__(self):
+        if self.n_heads < 1 or self.n_kv_heads < 1 or self.n_heads % self.n_kv_heads:
+            raise ValueError(f"n_heads {self.n_heads} is not a multiple of n_kv_heads {self.n_kv_heads}")
+        if not 1 <= self.head_dim <= 256 or not 1 <= self.v_dim <= 256:
+            raise ValueError(f"head sizes {self.head_dim} and {self.v_dim}: the attention kernels take up to 256")
+        if self.window is not None and self.window < 1:
+            raise ValueError("window must be at least 1")
+        if self.keep_first < 0:
+            raise ValueError("keep_first is not negative")
+        if self.value_blend not in (None, "first", "later"):
+            raise ValueError(f"value_blend {self.value_blend!r}: first, later or None")
+        if not self.scale > 0:
+            raise ValueError("scale must be positive")
+
+    @property
+    def cache_width(self) -> int:
+        """Elements per cached key and per cached value: the larger of the two sizes, padded to the
+        kernels' step."""
+        return (max(self.head_dim, self.v_dim) + 15) // 16 * 16
+
+
+@dataclass(frozen=True)
+class RetentionSpec:
+    """Linear attention with a fixed decay per head and no softmax or denominator: q, k [heads x
+    ``head_dim``] turned by ``position``, k scaled by head_dim^-1/2 after it, v [heads x ``v_dim``];
+    S <- decay_h S + k v^T, o = S^T q per head; each head's o over its root mean square (eps, no gain),
+    times silu(W_g x), then the output projection. The state is float32 and starts at zero."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    v_dim: int
+    decays: Tuple[float, ...]
+    eps: float
+    position: Optional[object] = None
+
+    def __post_init__(self):
+        if self.n_heads < 1 or len(self.decays) != self.n_heads:
+            raise ValueError(f"retention: {len(self.decays)} decays for {self.n_heads} heads")
+        if not 1 <= self.head_dim <= 256 or self.v_dim < 1:
+            raise ValueError(f"retention: heads of {self.head_dim} (1 to 256) and {self.v_dim}")
+
+
+@dataclass(frozen=True)
+class ReluSquaredSpec:
+    """y = Wd(relu(Wu x)^2), no bias."""
+    hidden: int
+    intermediate: int
+
+
+@dataclass(frozen=True)
+class RoutedExpertsSpec:
+    """A mixture of ``n_experts`` clamped gated feed-forwards (``expert``) of which a token uses ``top``.
+
+    Scores s = softmax(W_router x) in float32; the choice goes by s + ``correction`` (a stored vector;
+    ``corrected`` False: by s). Experts form ``n_groups`` equal groups of neighbours; a group's score is
+    its largest choice score, and only experts of the ``keep_groups`` best groups can be chosen. The
+    weights are the chosen experts' s over their sum (+ ``renorm_eps``). ``shared``: one more such
+    feed-forward that every token uses, added unweighted (None: none)."""
+    hidden: int
+    n_experts: int
+    top: int
+    expert: ClampedGLUSpec
+    n_groups: int = 1
+    keep_groups: int = 1
+    shared: Optional[ClampedGLUSpec] = None
+    corrected: bool = True
+    renorm_eps: float = 1e-20
+
+    def __post_init__(self):
+        if not 1 <= self.top <= self.n_experts:
+            raise ValueError(f"a token uses {self.top} of {self.n_experts} experts")
+        if self.n_groups < 1 or self.n_experts % self.n_groups or not 1 <= self.keep_groups <= self.n_groups:
+            raise ValueError(f"{self.n_experts} experts in {self.n_groups} groups, {self.keep_groups} kept")
+        if self.keep_groups * (self.n_experts // self.n_groups) < self.top:
+            raise ValueError(f"{self.keep_groups} groups of {self.n_experts // self.n_groups} experts hold fewer than {self.top}")
+
+
+@dataclass(frozen=True)
+class TokenSideSpec:
+    """A per-layer input that depends on the token alone: with e the layer's ``dim`` columns (from
+    ``index`` * dim on) of a table [vocab, ``n_layers`` * dim] that all layers share (``table_name``, a name
+    of the whole model), y = W_proj(gelu_tanh(W_gate x) * e) and x <- x + y / rms(y) * gain."""
+    hidden: int
+    dim: int
+    index: int
+    n_layers: int
+    vocab: int
+    eps: float
+    table_name: str = "side.embed"
+
+
+@dataclass(frozen=True)
 class BlockSpec:
     """One layer: which mixer, feed-forward and norms, how they are arranged,
     and the prefix its tensors carry on disk.
@@ -250,8 +371,11 @@ class BlockSpec:
     gate1: object = None
     gate2: object = None
     residual_mult: float = 1.0
+    # For the arrangement "prenorm_side": prenorm, then x <- x + side(x) on the stream itself (``side``
+    # None: none); ``ffn`` None: the layer has no feed-forward and no norm2.
+    side: object = None
 
-    ROLES = ("norm1", "mixer", "norm2", "ffn", "post_norm1", "post_norm2", "gate1", "gate2")
+    ROLES = ("norm1", "mixer", "norm2", "ffn", "post_norm1", "post_norm2", "gate1", "gate2", "side")
 
     def name_of(self, role: str) -> str:
         return self.prefix + dict(self.names)[role]

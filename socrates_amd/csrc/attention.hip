@@ -61,10 +61,13 @@ __device__ __forceinline__ void merge_partial(float& m, float& l, float (&a)[EPL
 //   softcap  > 0: the score becomes softcap * tanh(score / softcap) (after the bias)
 //   sinks    [Hq] float32: one more logit per head that takes its share of the softmax and
 //            contributes no value: the sum of weights gains exp(sinks[h] - max)
+//   keep_first  with a window: the keys at positions below keep_first stay visible to every later token,
+//            at their true positions (a token then walks those keys, then its window)
 struct ScoreTerms {
     float softcap;
     const float* sinks;
     const float* slopes;
+    int keep_first;
 };
 
 template <typename T, int GC>
@@ -81,8 +84,10 @@ paged_attn_token_kernel(const T* __restrict__ q, const T* __restrict__ k_pool,
     const int n = blockIdx.y, split = blockIdx.z;
     const int p = positions[n];
     const int lo = window > 0 ? max(0, p - window + 1) : 0;
-    const int start = lo + split * split_len;
-    const int end = min(p + 1, start + split_len);
+    const int kf = min(st.keep_first, lo);             // kept first keys that lie before the window
+    // the token's keys in the order they are walked: the kept first ones, then lo .. p
+    const int start = split * split_len;
+    const int end = min(kf + p + 1 - lo, start + split_len);
     if (start >= end) return;                          // this split holds no key of the token
 
     const int tid = threadIdx.x;
@@ -117,8 +122,8 @@ paged_attn_token_kernel(const T* __restrict__ q, const T* __restrict__ k_pool,
         float kx[KEYS_IN_FLIGHT][EPL], vx[KEYS_IN_FLIGHT][EPL];
 #pragma unroll
         for (int u = 0; u < KEYS_IN_FLIGHT; ++u) {
-            const int key = base + 16 * u;
-            if (key < end) {
+            if (base + 16 * u < end) {
+                const int key = base + 16 * u < kf ? base + 16 * u : base + 16 * u - kf + lo;
                 const int page = table[key / BS];
                 const size_t off = ((size_t)page * Hkv * BS + (size_t)(key % BS)) * D + head_off;
                 VecLoad<T, EPL>::load(k_pool + off, kx[u]);
@@ -134,7 +139,7 @@ paged_attn_token_kernel(const T* __restrict__ q, const T* __restrict__ k_pool,
 #pragma unroll
                     for (int e = 0; e < EPL; ++e) s = fmaf(qr[g][e], kx[u][e], s);
                     s = group16_sum(s);
-                    if (st.slopes) s += slope[g] * (float)(base + 16 * u - p);
+                    if (st.slopes) s += slope[g] * (float)((base + 16 * u < kf ? base + 16 * u : base + 16 * u - kf + lo) - p);
                     if (st.softcap > 0.f) s = st.softcap * tanhf(s / st.softcap);
                     const float mn = fmaxf(m[g], s);
                     const float alpha = soc_exp<T>(m[g] - mn);      // 0 on the first key (m = -inf)
@@ -211,7 +216,7 @@ __global__ void paged_attn_reduce_kernel(const float* __restrict__ part_o,
     const int h = blockIdx.x, n = blockIdx.y;
     const int p = positions[n];
     const int lo = window > 0 ? max(0, p - window + 1) : 0;
-    const int np = min(n_splits, (p + 1 - lo + split_len - 1) / split_len);
+    const int np = min(n_splits, (min(st.keep_first, lo) + p + 1 - lo + split_len - 1) / split_len);
     const size_t base = ((size_t)n * Hq + h) * n_splits;
     float M = st.sinks ? st.sinks[h] : -INFINITY;
     for (int s = 0; s < np; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
@@ -260,18 +265,19 @@ static int dispatch_token(int G, const void* q, const void* k_pool, const void* 
 
 // q [N, Hq, D]; pools [pages, Hkv, BS, D]; out [N, Hq, D]. window <= 0: no window.
 // n_splits > 1 needs part_o [N, Hq, n_splits, D] and part_ml [N, Hq, n_splits, 2] (float32);
-// split s covers keys lo + s * split_len .. of each token. softcap (0: none), sinks and slopes
-// ([Hq] float32 each, or null): see ScoreTerms. Any scale, also none or a negative one.
+// split s covers the keys s * split_len .. of each token's walk (the kept first keys, then its window).
+// softcap (0: none), sinks and slopes ([Hq] float32 each, or null) and keep_first (0: none): see
+// ScoreTerms. Any scale, also none or a negative one.
 SOC_EXPORT int soc_paged_attention_tokens(const void* q, const void* k_pool, const void* v_pool,
                                           const int* block_table, int table_width,
                                           const int* token_rows, const int* positions, void* out,
                                           float* part_o, float* part_ml, int N, int Hq, int Hkv,
                                           int BS, float scale, int window, int split_len,
                                           int n_splits, int dtype, float softcap, const float* sinks,
-                                          const float* slopes, hipStream_t stream) {
+                                          const float* slopes, int keep_first, hipStream_t stream) {
     if (N <= 0) return 0;
-    if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || split_len < 1 || softcap < 0.f) return (int)hipErrorInvalidValue;
-    const ScoreTerms st{softcap, sinks, slopes};
+    if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || split_len < 1 || softcap < 0.f || keep_first < 0) return (int)hipErrorInvalidValue;
+    const ScoreTerms st{softcap, sinks, slopes, window > 0 ? keep_first : 0};
     if (n_splits > 1 && (!part_o || !part_ml)) return (int)hipErrorInvalidValue;
     if (N > 65535 || n_splits > 65535) return (int)hipErrorInvalidValue;
     const int G = Hq / Hkv;

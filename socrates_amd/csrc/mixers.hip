@@ -12,6 +12,7 @@
 // seq_qstart [S + 1] gives each sequence's tokens among the step's, seq_rows [S] its row of
 // the state tensor [rows, stride] (float32).
 #include "common.h"
+#include "recurrent.h"
 
 __device__ __forceinline__ float soc_sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
 
@@ -350,25 +351,6 @@ SOC_EXPORT int soc_wkv_decay(const float* t, const void* w2, const float* w0, fl
 // else 64). Tokens go in batches: what all threads need of a batch (per key: r, k, decay; or B,
 // C) is staged through LDS; the next batch's global loads are issued before the current batch is computed
 // and land in LDS after it; the partial sums of a column's PARTS threads meet in LDS once per batch.
-// (tokens per batch: 16 for states of up to 64 keys, else 8: what LDS holds twice over)
-constexpr int rec_batch(int keys) { return keys <= 64 ? 16 : 8; }
-
-// A barrier for threads that meet in LDS only: a wave waits for its own LDS accesses, not for its global
-// loads and stores in flight (__syncthreads waits for those too, which would drain the next batch's
-// loads, issued on purpose before the current batch is computed, at every barrier).
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
-#define SOC_BY_STATE_SIZE(D, CALL)                                         \
-    switch (((D) + 15) / 16) {                                              \
-        case 1: CALL(16); break;   case 2: CALL(32); break;                 \
-        case 3: CALL(48); break;   case 4: CALL(64); break;                 \
-        case 5: case 6: CALL(96); break;                                    \
-        case 7: case 8: CALL(128); break;                                   \
-        case 9: case 10: case 11: case 12: CALL(192); break;                \
-        case 13: case 14: case 15: case 16: CALL(256); break;               \
-        default: return (int)hipErrorInvalidValue;                          \
-    }
-
 // Decay per key channel: o_t[j] = sum_i r_t[i] (S[i, j] + u[i] k_t[i] v_t[j]); S[i, j] <- w_t[i] S[i, j] +
 // k_t[i] v_t[j]. o goes out in float32; its norm over the head is another kernel's.
 template <typename T, int DK, int CW>
@@ -467,13 +449,6 @@ static void launch_wkv(const void* r, const void* k, const void* v, const float*
     hipLaunchKernelGGL((wkv_kernel<T, DK, CW>), dim3(H * ((D + CW - 1) / CW), n_seqs), dim3(256), 0, stream, (const T*)r, \
                        (const T*)k, (const T*)v, decay, bonus, H, D, state, (size_t)stride, offset, seq_qstart, seq_rows, out)
     if (cw == 16) SOC_WKV_LAUNCH(16); else SOC_WKV_LAUNCH(64);
-}
-
-// Columns per workgroup: 64, or 16 where heads and sequences alone leave most compute units idle.
-// (A step with a prompt portion in it is as long as that portion's walk, whatever else is in the step.)
-static int columns_per_workgroup(int H, int cols, int n_seqs, int max_q_len) {
-    if (max_q_len > 64) return 16;
-    return (long long)H * ((cols + 63) / 64) * n_seqs >= 192 ? 64 : 16;
 }
 
 SOC_EXPORT int soc_wkv(const void* r, const void* k, const void* v, const float* decay, const float* bonus, int H, int D,

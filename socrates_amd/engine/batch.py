@@ -55,6 +55,9 @@ class StepContext:
     max_ctx_len: int
     host: dict = field(default_factory=dict)
     upload: object = None        # int32 numpy array -> device tensor, for kernels that plan on the host
+    # what one layer leaves for a later layer of the same step (the first blended layer's values, say); a
+    # layer writes its entry before any layer reads it, in every step
+    carry: dict = field(default_factory=dict)
 
 
 def build_context(entries: List[StepEntry], starts: Sequence[int], device, vocab_size=None,

@@ -11,7 +11,8 @@ This module holds the class, its switches and thresholds, and the small kernels 
 norms, sampling); ``products.py`` the matrix products in all their forms, ``attention.py``
 attention and what prepares it, ``planning.py`` the host arithmetic of key splits,
 ``mixers.py`` the mixers with a state per row, attention over a cached latent and blocks with norms
-on both sides of a branch, ``common.py`` what they share, ``build.py`` the compiler and loader.
+on both sides of a branch, ``hybrid.py`` attention whose keys and values differ in size, retention, routed
+experts and a per-token side input, ``common.py`` what they share, ``build.py`` the compiler and loader.
 """
 
 from __future__ import annotations
@@ -22,6 +23,7 @@ from ctypes import c_float, c_int, c_longlong, c_void_p
 import torch
 
 from .attention import Attention
+from .hybrid import Hybrid
 from .mixers import Mixers
 from .build import KernelBuildError, build_all, compile_library, load_library
 from .common import (_ATTENTION_SIGNATURES, _DTYPE_CODE, _EW_SIGNATURES, _GEMM_SIGNATURES, _SAMPLING_SIGNATURES, KernelError,
@@ -33,7 +35,7 @@ __all__ = ["HipKernels", "KernelBuildError", "KernelError", "MAX_KEY_SPLITS", "N
            "compile_library", "load_library", "plan_key_splits"]
 
 
-class HipKernels(Products, Attention, Mixers):
+class HipKernels(Products, Attention, Mixers, Hybrid):
     def __init__(self, dtype=torch.bfloat16, device="cuda:0"):
         if dtype not in _DTYPE_CODE:
             raise ValueError(f"compute dtype must be float32 or bfloat16, not {dtype}")

@@ -275,7 +275,8 @@ class Attention:
         what an architecture adds to plain softmax attention, a dict with any of ``softcap``
         (float: scores become softcap * tanh(scores / softcap)), ``sinks`` (float32 [Hq]: one
         more logit per head in the softmax's sum, with no value) and ``slopes`` (float32 [Hq]:
-        slope * (key position - query position) added to the scaled scores). Such a layer,
+        slope * (key position - query position) added to the scaled scores) and ``keep_first``
+        (int, with a window: the keys at positions below it stay visible to every later token). Such a layer,
         and one whose scale is not positive, goes to the kernel that computes scores on the
         vector units, in either dtype; the MFMA kernels take plain scores only."""
         N, Hq, D = q.shape
@@ -290,18 +291,22 @@ class Attention:
         out = torch.empty((N, Hq * D), dtype=self.dtype, device=self.device)
         w = int(window) if window else 0
         G = Hq // Hkv
-        softcap, sinks, slopes = 0.0, None, None
+        softcap, sinks, slopes, keep_first = 0.0, None, None, 0
         if terms:
-            if set(terms) - {"softcap", "sinks", "slopes"}:
-                raise KernelError(f"attention: unknown score terms {sorted(set(terms) - {'softcap', 'sinks', 'slopes'})}")
+            known = {"softcap", "sinks", "slopes", "keep_first"}
+            if set(terms) - known:
+                raise KernelError(f"attention: unknown score terms {sorted(set(terms) - known)}")
             softcap = float(terms.get("softcap") or 0.0)
+            keep_first = int(terms.get("keep_first") or 0) if w else 0
+            if keep_first < 0:
+                raise KernelError("attention: the number of first keys that stay visible is not negative")
             sinks, slopes = terms.get("sinks"), terms.get("slopes")
             if softcap < 0:
                 raise KernelError("attention: a soft cap is positive")
             for name, t in (("sinks", sinks), ("slopes", slopes)):
                 if t is not None:
                     self._want(t, name, torch.float32, (Hq,))
-        plain = softcap == 0.0 and sinks is None and slopes is None and scale > 0
+        plain = softcap == 0.0 and sinks is None and slopes is None and scale > 0 and keep_first == 0
         if self.dtype == torch.bfloat16 and self.attention_mfma and plain:
             gpl = max(0, (min(G, 16) - 1).bit_length())
             decode = getattr(ctx, "max_q_len", 1) == 1
@@ -370,7 +375,7 @@ class Attention:
             self.last_attention_kernel = ("wave", rt)
             self._wave_attention(lib, q, slot, ctx, out, scale, w, rt, gpl, None)
             return out
-        max_keys = ctx.max_ctx_len if not w else min(w, ctx.max_ctx_len)
+        max_keys = ctx.max_ctx_len if not w else min(w + keep_first, ctx.max_ctx_len)
         split_len, n_splits = self.plan_splits(N, Hkv, G, max_keys)
         part_o = part_ml = None
         if n_splits > 1:
@@ -387,5 +392,5 @@ class Attention:
                 _ptr(part_ml[lo:lo + n]) if part_ml is not None else None,
                 c_int(n), c_int(Hq), c_int(Hkv), c_int(slot.block_size), c_float(scale), c_int(w),
                 c_int(split_len), c_int(n_splits), c_int(self.code), c_float(softcap), _ptr(sinks), _ptr(slopes),
-                self._stream()), "paged_attention")
+                c_int(keep_first), self._stream()), "paged_attention")
         return out

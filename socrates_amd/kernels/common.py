@@ -65,9 +65,21 @@ _MIXER_SIGNATURES = {
     "soc_latent_query_turn": [P, I, I, I, I, I, I, P, I, P, P, I, P],
     "soc_head_linear": [P, I, P, P, I, I, I, I, I, I, P],
 }
+_HYBRID_SIGNATURES = {
+    "soc_attn_prepare": [P, I, I, I, I, P, I, P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
+    "soc_head_gate": [P, P, I, P, I, I, I, I, I, P],
+    "soc_retention": [P, I, I, I, I, P, P, I, F, P, I, I, I, P, L, I, P, P, P, I, I, I, P],
+    "soc_relu_squared": [P, P, L, I, P],
+    "soc_moe_route": [P, P, I, I, I, I, I, F, P, P, P],
+    "soc_moe_sort": [P, I, I, I, I, P, P, P, P, P],
+    "soc_grouped_linear": [P, I, P, I, P, P, P, I, P, I, I, I, F, F, I, I, P],
+    "soc_moe_combine": [P, P, P, P, P, I, I, I, I, P],
+    "soc_side_gate": [P, P, I, I, P, I, P, I, I, I, P],
+    "soc_add_cast": [P, P, P, I, L, P, I, P],
+}
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P, P, P, I, I, I, P]}
 _ATTENTION_SIGNATURES = {
-    "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, F, P, P, P],
+    "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, F, P, P, I, P],
     "soc_paged_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, I, I, I, P],
     "soc_paged_attention_prefill": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, F, I, I, I, P],
     "soc_paged_attention_decode_fused": [P, I, P, P, P, I, P, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P, P, P, F, I, I, P],

@@ -32,7 +32,10 @@ def block_tensors(spec: BlockSpec):
 
 def _joined(base: str, local: str) -> str:
     """A part's tensor on disk: the part's name, a dot, the local name; a local name of ""
-    is the tensor that carries the part's own name."""
+    is the tensor that carries the part's own name, and one that starts with "/" is a name of the
+    whole model (a tensor that several layers share)."""
+    if local.startswith("/"):
+        return local[1:]
     return f"{base}.{local}" if local else base
 
 
@@ -175,5 +178,43 @@ class SandwichBlock:
         return None if h is None else Normed(h)
 
 
+class SideInputBlock:
+    """Prenorm with a per-layer side input at the end: x <- x + mixer(norm1(x)); x <- x + ffn(norm2(x)) (a
+    layer may have no feed-forward); then, if the layer has one, x <- x + norm(side(x)) with side reading the
+    stream itself. The sum before the side input, and the stream in the compute dtype, are one kernel; the
+    norm of the side's result, its sum into the stream and the next block's first norm another."""
+    chains = True
+
+    def __init__(self, spec: BlockSpec, weights, ops):
+        self.spec, self.ops = spec, ops
+        for role in ("norm1", "mixer", "norm2", "ffn", "side"):
+            sub = getattr(spec, role)
+            setattr(self, role, None if sub is None else build_part(sub, _sub_tensors(spec, role, weights), ops))
+        if self.ffn is not None and self.norm2 is None:
+            raise ValueError("a feed-forward needs the norm before it")
+        parts = (self.norm1, self.mixer, self.norm2, self.ffn, self.side)
+        self.capturable = all(getattr(p, "capturable", True) for p in parts if p is not None)
+
+    def reserve(self, n_positions):
+        for part in (self.norm1, self.mixer, self.norm2, self.ffn, self.side):
+            if hasattr(part, "reserve"):
+                part.reserve(n_positions)
+
+    def forward(self, residual, pending, ctx, slot, write=True, nxt=None):
+        ops = self.ops
+        h = pending.rows if isinstance(pending, Normed) else self.norm1.add_norm(residual, pending)
+        out = self.mixer.forward(h, ctx, slot, write)
+        if self.ffn is not None:
+            out = self.ffn.forward(self.norm2.add_norm(residual, out), ctx)
+        if self.side is None:
+            return out
+        y = self.side.forward(ops.add_cast(residual, out), ctx)
+        first_of_next = getattr(nxt, "norm1", None)
+        follows = first_of_next.fusable() if hasattr(first_of_next, "fusable") else None
+        rows = ops.gated_norm_add(residual, y, None, None, self.side.gain, self.side.eps, 1.0, *(follows or (None, 0.0)))
+        return None if rows is None else Normed(rows)
+
+
 register_arrangement("prenorm", PreNormBlock)
+register_arrangement("prenorm_side", SideInputBlock)
 register_arrangement("sandwich", SandwichBlock)

@@ -5,7 +5,7 @@ from __future__ import annotations
 
 import torch
 
-from ..config.specs import ClampedGLUSpec, SigmoidGateSpec, SwiGLUSpec
+from ..config.specs import ClampedGLUSpec, ReluSquaredSpec, SigmoidGateSpec, SwiGLUSpec
 from .registry import TensorDecl, register_part
 
 
@@ -75,6 +75,21 @@ class ClampedGLU:
         return (y, both[:, 2 * ff:]) if self.adopted else y
 
 
+class ReluSquared:
+    """y = Wd(relu(Wu x)^2)."""
+
+    @staticmethod
+    def tensors(spec: ReluSquaredSpec):
+        return {"up": TensorDecl((spec.intermediate, spec.hidden)), "down": TensorDecl((spec.hidden, spec.intermediate))}
+
+    def __init__(self, spec: ReluSquaredSpec, tensors, ops):
+        self.spec, self.ops = spec, ops
+        self.w_up, self.w_down = tensors["up"], tensors["down"]
+
+    def forward(self, x, ctx=None):
+        return self.ops.linear(self.ops.relu_squared(self.ops.linear(x, self.w_up)), self.w_down)
+
+
 class SigmoidGate:
     """Holds W [dim, dim] and b [dim] of sigmoid(W h + b); the block computes it where it closes
     a branch."""
@@ -90,3 +105,4 @@ class SigmoidGate:
 register_part(SwiGLUSpec, SwiGLU)
 register_part(ClampedGLUSpec, ClampedGLU)
 register_part(SigmoidGateSpec, SigmoidGate)
+register_part(ReluSquaredSpec, ReluSquared)

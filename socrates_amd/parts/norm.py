@@ -15,11 +15,11 @@ from .registry import TensorDecl, register_part
 class RMSNorm:
     @staticmethod
     def tensors(spec: RMSNormSpec):
-        return {"weight": TensorDecl((spec.dim,), "vector")}
+        return {spec.tensor: TensorDecl((spec.dim,), "vector")}
 
     def __init__(self, spec: RMSNormSpec, tensors, ops):
         self.spec, self.ops = spec, ops
-        self.weight = tensors["weight"]
+        self.weight = tensors[spec.tensor]
 
     free_layout = True      # add_norm takes ``by_tile``
 

@@ -61,10 +61,13 @@ class TensorDecl:
 
 @dataclass(frozen=True)
 class PagedKV:
-    """A mixer that keeps keys and values of every position (or a window of them) in pages."""
+    """A mixer that keeps keys and values of every position (or a window of them) in pages.
+    ``keep_first``: with a window, the positions below it stay visible to every later token, so
+    the pages that hold them are never given back before the row closes."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    keep_first: int = 0
 
 
 @dataclass(frozen=True)

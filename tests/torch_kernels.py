@@ -128,7 +128,8 @@ class TorchKernels:
     def paged_attention(self, q, slot, ctx, scale, window, terms=None):
         """Token by token: gather the row's keys 0..p through the table, mask the window.
         ``terms``: a bias by distance (``slopes`` [Hq]), a soft cap of the scores, one more
-        logit per head in the softmax's sum (``sinks`` [Hq])."""
+        logit per head in the softmax's sum (``sinks`` [Hq]), first keys that stay visible
+        behind a window (``keep_first``)."""
         terms = terms or {}
         N, Hq, D = q.shape
         Hkv, bs = slot.k.shape[1], slot.block_size
@@ -141,6 +142,8 @@ class TorchKernels:
             p, row = int(positions[t]), int(rows[t])
             lo = 0 if window is None else max(0, p - window + 1)
             idx = np.arange(lo, p + 1)
+            if window is not None and terms.get("keep_first"):
+                idx = np.concatenate([np.arange(0, min(int(terms["keep_first"]), lo)), idx])
             pages = torch.as_tensor(table[row, idx // bs].astype(np.int64), device=q.device)
             offs = torch.as_tensor(idx % bs, device=q.device)
             k = slot.k[pages, :, offs].to(self.acc)          # [n, Hkv, D]
@@ -249,14 +252,16 @@ class TorchKernels:
             state[row, offset:offset + H * Ns * P] = S.reshape(-1).to(state.dtype)
         return out.reshape(N, inner).to(torch.float32 if A == torch.float32 else A)
 
-    def gated_group_norm(self, y, z, gain, groups, eps):
+    def gated_group_norm(self, y, z, gain, groups, eps, gate_first=True):
         A = self.acc
         N, inner = y.shape
         zz = z[:, :inner].to(A)
-        y = y.to(A) * (zz * torch.sigmoid(zz))
+        gate = zz * torch.sigmoid(zz)
+        y = y.to(A) * gate if gate_first else y.to(A)
         y = y.view(N, groups, inner // groups)
         y = y / torch.sqrt(y.pow(2).mean(-1, keepdim=True) + eps)
-        return (y.reshape(N, inner) * gain.to(A)).to(self.dtype)
+        y = y.reshape(N, inner) * gain.to(A)
+        return (y if gate_first else y * gate).to(self.dtype)
 
     # -- attention over a cached latent ------------------------------------------------------------
     def _turn_pairs(self, x, positions, inv_freq):
@@ -299,6 +304,116 @@ class TorchKernels:
         H, n_out, K = w.shape
         y = torch.einsum("nhk,hok->nho", x[..., :K].to(self.acc), w.to(self.acc))
         return y.reshape(x.shape[0], H * n_out).to(self.dtype)
+
+    # -- attention whose keys and values differ in size, retention, routed experts, side input --------
+    def attn_prepare(self, x, cols, Hq, Hkv, D, Dv, P, q_gain, k_gain, eps, inv_freq, rotary_dim, positions,
+                     token_rows, slot, first=None, lam=None):
+        A = self.acc
+        N = x.shape[0]
+        cq, ck, cv = cols
+        q = x[:, cq:cq + Hq * D].reshape(N, Hq, D).to(A)
+        k = x[:, ck:ck + Hkv * D].reshape(N, Hkv, D).to(A)
+        if q_gain is not None:
+            q, k = self._norm(q, q_gain, eps), self._norm(k, k_gain, eps)
+        if rotary_dim:
+            q = self._rotate(q, positions, inv_freq, rotary_dim)
+            if Hkv:
+                k = self._rotate(k, positions, inv_freq, rotary_dim)
+        out = torch.zeros((N, Hq, P), dtype=self.dtype, device=x.device)
+        out[..., :D] = q.to(self.dtype)
+        if slot is not None and Hkv:
+            v = x[:, cv:cv + Hkv * Dv].to(A)
+            if first is not None:
+                l = lam.to(A).reshape(())
+                v = (1.0 - l) * v + l * first.to(A)
+            kp = torch.zeros((N, Hkv, P), dtype=slot.k.dtype, device=x.device)
+            vp = torch.zeros((N, Hkv, P), dtype=slot.v.dtype, device=x.device)
+            kp[..., :D] = k.to(slot.k.dtype)
+            vp[..., :Dv] = v.reshape(N, Hkv, Dv).to(slot.v.dtype)
+            self.kv_write(kp, vp, positions, token_rows, slot)
+        return out
+
+    def head_gate(self, o, H, P, Dv, gate):
+        N = o.shape[0]
+        y = o.view(N, H, P)[..., :Dv].to(self.acc)
+        if gate is not None:
+            y = y * torch.sigmoid(gate.to(self.acc)).unsqueeze(-1)
+        return y.reshape(N, H * Dv).to(self.dtype)
+
+    def retention(self, x, cols, H, D, Dv, inv_freq, rotary_dim, k_scale, decays, state, offset, ctx):
+        A = self.acc
+        N = x.shape[0]
+        cq, ck, cv = cols
+        q = x[:, cq:cq + H * D].reshape(N, H, D).to(A)
+        k = x[:, ck:ck + H * D].reshape(N, H, D).to(A)
+        v = x[:, cv:cv + H * Dv].reshape(N, H, Dv).to(A)
+        if rotary_dim:
+            q = self._rotate(q, ctx.positions, inv_freq, rotary_dim)
+            k = self._rotate(k, ctx.positions, inv_freq, rotary_dim)
+        k = k * k_scale
+        out = torch.empty((N, H, Dv), dtype=A, device=x.device)
+        for row, lo, hi in self._sequences(ctx):
+            S = state[row, offset:offset + H * D * Dv].to(A).view(H, D, Dv).clone()
+            for t in range(lo, hi):
+                S = decays.to(A).view(H, 1, 1) * S + k[t].unsqueeze(-1) * v[t].unsqueeze(-2)
+                out[t] = torch.einsum("hk,hkv->hv", q[t], S)
+            state[row, offset:offset + H * D * Dv] = S.reshape(-1).to(state.dtype)
+        return out.reshape(N, H * Dv).to(torch.float32 if A == torch.float32 else A)
+
+    def relu_squared(self, x):
+        return (torch.relu(x.to(self.acc)) ** 2).to(self.dtype)
+
+    def moe_route(self, logits, correction, top, n_groups=1, keep_groups=1, renorm_eps=1e-20):
+        A = self.acc
+        s = torch.softmax(logits.to(A), dim=-1)
+        c = s if correction is None else s + correction.to(A)
+        N, E = s.shape
+        if n_groups > 1 and keep_groups < n_groups:
+            per = E // n_groups
+            best = c.view(N, n_groups, per).max(-1).values
+            kept = torch.zeros((N, n_groups), dtype=torch.bool, device=s.device)
+            for _ in range(keep_groups):                      # the lower index among equals
+                g = torch.where(kept, torch.full_like(best, -float("inf")), best).argmax(-1)
+                kept[torch.arange(N), g] = True
+            c = torch.where(kept.repeat_interleave(per, dim=1), c, torch.full_like(c, -float("inf")))
+        idx = torch.empty((N, top), dtype=torch.int64, device=s.device)
+        taken = torch.zeros_like(c, dtype=torch.bool)
+        for r in range(top):
+            e = torch.where(taken, torch.full_like(c, -float("inf")), c)
+            # argmax returns the first of equal maxima only by convention; make it so
+            m = e.max(-1, keepdim=True).values
+            first = (e == m).to(torch.int64).argmax(-1)
+            idx[:, r] = first
+            taken[torch.arange(N), first] = True
+        w = torch.gather(s, 1, idx)
+        w = w / (w.sum(-1, keepdim=True) + renorm_eps)
+        return idx.to(torch.int32), w.to(torch.float32 if A == torch.float32 else A)
+
+    def moe_experts(self, x, idx, weight, w_gate_up, w_down, limit, slope, extra=None):
+        A = self.acc
+        N, top = idx.shape
+        ff = w_gate_up.shape[1] // 2
+        out = torch.zeros((N, w_down.shape[1]), dtype=A, device=x.device)
+        if extra is not None:
+            out += extra.to(A)
+        for r in range(top):
+            e = idx[:, r].long()
+            both = torch.einsum("nk,nok->no", x.to(A), w_gate_up[e].to(A)).to(self.dtype)
+            act = self.glu_clamped(both, limit, slope, ff)
+            y = torch.einsum("nk,nok->no", act.to(A), w_down[e].to(A))
+            out += weight[:, r:r + 1].to(A) * y
+        return out.to(torch.float32 if A == torch.float32 else A)
+
+    def side_gate(self, t, table, col0, token_ids):
+        z = t.to(self.acc)
+        g = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        e = table[token_ids.long(), col0:col0 + t.shape[1]].to(self.acc)
+        return (g * e).to(self.dtype)
+
+    def add_cast(self, residual, delta):
+        if delta is not None:
+            residual += (delta.sum(0) if delta.dim() == 3 else delta).to(residual.dtype)
+        return residual.to(self.dtype)
 
     # -- sampling ----------------------------------------------------------------------------
     def argmax(self, logits):
