@@ -97,7 +97,7 @@ def route(h, W, r):
     s = torch.softmax(h @ W["router"].T, dim=-1)
     choice = s + W["correction"]
     T, E = s.shape
-    groups = r["groups"]
+    groups = r.get("groups") or {"count": 1, "keep": 1}
     per = E // groups["count"]
     best = choice.view(T, groups["count"], per).max(-1).values
     kept = best.topk(groups["keep"], dim=-1).indices
