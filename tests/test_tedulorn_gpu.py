@@ -23,8 +23,11 @@ pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parents[1]
 DEV = "cuda:0"
 DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
-# in units of the logits' spread per position
-TOL = {"float32": 3e-4, "bfloat16": (0.2, 0.05)}
+# in units of the logits' spread per position; bfloat16: (every row, nine rows in ten). A token whose choice of
+# experts hangs on less than bfloat16 resolves may choose otherwise than the plain model, and its row then
+# differs by a good part of the spread: the limit for every row leaves room for that, the limit for nine rows in
+# ten is what a fault of a window, a state, a page or a kernel cannot keep.
+TOL = {"float32": 3e-4, "bfloat16": (0.6, 0.05)}
 
 
 @pytest.fixture(scope="module")
@@ -246,18 +249,18 @@ def test_drawn_configurations(tmp_path, kernel_sets, seed, dtype):
 
 @pytest.mark.parametrize("dtype", list(DTYPES))
 def test_a_wider_model_with_long_prompts(tmp_path, kernel_sets, dtype):
-    """Width 320, five layers, keys of 80 beside values of 48, a state of 64 x 96, twenty experts in four groups,
+    """Width 320, five layers, keys of 80 beside values of 48 and of 32 beside 112, a state of 64 x 96, twenty experts in four groups,
     windows of 100 and 37 with 6 and 0 kept first tokens, prompts of up to 700 tokens: decoded at the end, mixed,
     and in portions of 2 to 200 tokens, through captured decode steps."""
     cfg = model(320, 500, [attention(10, 5, 80, 48, window=100, keep_first=6, scale=0.1, rot=40), retention(5, 64, 96, (0.9, 0.97, 0.99, 0.995, 0.999)),
-                           attention(4, 1, 32, 240, window=37, keep_first=0, scale=0.2, v_mix=False),
+                           attention(4, 1, 32, 112, window=37, keep_first=0, scale=0.2, v_mix=False),
                            attention(5, 5, 64, 48, window=300, keep_first=20, scale=0.12, base=1e6), retention(2, 128, 32, (0.98, 0.9), rot=64)],
                 [moe(20, 4, 64, 1.0, groups=(4, 2), shared=(96, 1.5)), dense(520), moe(7, 2, 100, 2.0), None, moe(16, 1, 32, 0.8, groups=(8, 3))],
                 side=12, scale=4.0)
     folder = write_model(tmp_path / "m", cfg, seed=5)
     prompts = random_prompts([700, 333, 64, 150], cfg["vocab"], seed=6)
     want = oracle(folder, prompts)
-    tol = TOL[dtype] if dtype == "float32" else (0.25, 0.06)
+    tol = TOL[dtype] if dtype == "float32" else (0.6, 0.06)
     for name, steps in (("tail", trace_tail_decode(prompts, 40)), ("mixed", trace_mixed(prompts, seed=7)),
                         ("portions", trace_portions(prompts, seed=8, sizes=(2, 3, 64, 65, 128, 200)))):
         runner = make_runner(folder, kernel_sets[dtype], max_rows=4, max_len=768, block_size=16, num_blocks=4 * 48)
