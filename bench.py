@@ -298,6 +298,75 @@ def mitisun_beside_qwen3(args, dtype, item):
     return 0
 
 
+def tedulorn_dict(width, ff, n_layers, heads, kv_heads, window=1024):
+    """A Tedulorn of ``n_layers`` layers at a real model's layer sizes: two layers of windowed attention (heads of
+    128, the first four tokens kept, values blended) and one of retention (heads of 128 x 128) in turn; the first
+    layer's feed-forward dense, the others 32 experts of a quarter of the dense size in four groups, four per token
+    from two groups, beside a shared one; a side input of 64 per token and layer."""
+    attention = {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                 "rot": {"base": 1000000.0, "dims": 64}, "mask": {"size": window, "keep_first": 4}, "v_mix": True}
+    n_ret = width // 128
+    kinds = [{"type": "attention", "mixer": attention}, {"type": "attention", "mixer": attention},
+             {"type": "retention", "mixer": {"heads": n_ret, "dim": 128, "vdim": 128, "rot": {"base": 10000.0, "dims": 128},
+                                             "decay": [1.0 - 2.0 ** (-5 - 4 * h / n_ret) for h in range(n_ret)]}}]
+    moe = {"kind": "moe", "expert": {"ff": ff // 4, "limit": 7.0}, "shared": {"ff": ff // 4, "limit": 7.0},
+           "router": {"experts": 32, "top": 4, "groups": {"count": 4, "keep": 2}}}
+    layers = []
+    for i in range(n_layers):
+        layer = json.loads(json.dumps(kinds[i % 3]))
+        layer["mlp"] = {"kind": "dense", "ff": ff} if i == 0 else json.loads(json.dumps(moe))
+        layers.append(layer)
+    return {"architecture": "Tedulorn", "vocab": 151936, "width": width, "layers": layers, "norm": {"eps": 1e-6},
+            "embedding": {"scale": 1.0}, "token_side": {"dim": 64}}
+
+
+def tedulorn_beside_others(args, dtype, item):
+    """Prefill and decode of Tedulorn at a few real layer sizes, beside Mitisun (the other model of mixed layers)
+    and Qwen3 of the same width, feed-forward size, vocabulary and number of layers, all with the library's default
+    solutions for its products. One JSON line of its own; the default workload and its line are untouched."""
+    import torch
+    sizes = [("4b", "qwen3-4b", dict(wkv_heads=40, ssm_heads=80, attn_heads=20)),
+             ("8b", "qwen3-8b", dict(wkv_heads=64, ssm_heads=128, attn_heads=32))]
+    n_layers = args.layers or 12
+    out = {"metric": "prefill and decode of Tedulorn beside Mitisun and Qwen3 at equal width, feed-forward, vocabulary and layers",
+           "dtype": args.dtype, "layers": n_layers, "batch": args.batch, "context": args.context,
+           "prefill_tokens": args.prefill_tokens, "data": "synthetic: seeded random weights, uniform random token ids",
+           "sizes": {}}
+    only = set(filter(None, (args.only or "").split(",")))
+    for tag, preset, heads in sizes:
+        if only and tag not in only:
+            continue
+        q = preset_dict(preset)
+        q["num_hidden_layers"] = n_layers
+        m = mitisun_dict(q["hidden_size"], q["intermediate_size"], n_layers, **heads)
+        t = tedulorn_dict(q["hidden_size"], q["intermediate_size"], n_layers, q["num_attention_heads"], q["num_key_value_heads"])
+        point = {}
+        for name, cfg in (("tedulorn", t), ("mitisun", m), ("qwen3", q)):
+            if only & {"tedulorn", "mitisun", "qwen3"} and name not in only:
+                continue
+            config, engine = build_engine(cfg, dtype, args.batch, args.max_len, seed=0, compile_=not args.no_graphs,
+                                          chunk=max(2048, args.prefill_tokens), block_size=args.block_size)
+            V = cfg.get("vocab_size") or cfg["vocab"]
+            tok_s, ms = decode_rate(engine, args.batch, args.context, args.steps, args.warmup, V, seed=1)
+            pre_s = prefill_rate(engine, args.prefill_tokens, V, seed=2)
+            weights = config.param_counts()["read_per_step"] * item
+            if name == "tedulorn":
+                # of the experts a step of several tokens reads what its tokens chose: at most all, at least a token's share
+                weights = config.step_weight_bytes(args.batch, item)
+            cache = (args.batch * args.context * config.kv_bytes_per_token(item) if name == "qwen3"
+                     else config.step_cache_bytes(args.batch, args.context, item))
+            point[name] = {"decode_tok_s": round(tok_s, 1), "decode_ms": round(ms, 4),
+                           "decode_hbm_frac": round((weights + cache) / (ms * 1e-3) / 1e9 / HBM_GBPS, 4),
+                           "prefill_ms": round(pre_s * 1e3, 3), "prefill_tok_s": round(args.prefill_tokens / pre_s, 1),
+                           "prefill_flop_frac": round(config.prefill_flops(args.prefill_tokens) / pre_s / PEAK_FLOPS[args.dtype], 4),
+                           "weights_gb": round(weights / 1e9, 3)}
+            release(engine)
+            torch.cuda.synchronize()
+        out["sizes"][tag] = point
+    print(json.dumps(out))
+    return 0
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -317,6 +386,10 @@ def main(argv=None):
     ap.add_argument("--mitisun", action="store_true",
                     help="instead of the default workload: prefill and decode of Mitisun at 4B- and 8B-sized layers "
                          "(--layers of them, default 12), each beside Qwen3 of the same sizes")
+    ap.add_argument("--tedulorn", action="store_true",
+                    help="instead of the default workload: prefill and decode of Tedulorn at 4B- and 8B-sized layers "
+                         "(--layers of them, default 12), each beside Mitisun and Qwen3 of the same sizes")
+    ap.add_argument("--only", default=None, help="--tedulorn: sizes and models to run, with commas (4b,8b,tedulorn,mitisun,qwen3)")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per page of the cache (the reference's 16)")
     ap.add_argument("--no-graphs", action="store_true")
@@ -346,6 +419,8 @@ def main(argv=None):
     item = 2 if args.dtype == "bf16" else 4
     if args.mitisun:
         return mitisun_beside_qwen3(args, dtype, item)
+    if args.tedulorn:
+        return tedulorn_beside_others(args, dtype, item)
     if args.mixed:
         args.preset = args.preset or MIXED_PRESET
         args.max_len = max(args.max_len, 8192)

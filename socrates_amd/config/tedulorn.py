@@ -251,6 +251,25 @@ class TedulornConfig:
             per_step += n * next((f for p, f in share.items() if name.startswith(p)), 1.0)
         return {"total": total, "read_per_step": int(per_step)}
 
+    def step_weight_bytes(self, batch: int, item: int) -> int:
+        """Bytes of weights that a decode step of ``batch`` tokens reads if its tokens choose their experts
+        independently and evenly: of E experts, E (1 - (1 - top / E)^batch) on average."""
+        from ..parts import expected_tensors
+        plan = self.plan()
+        share = {}
+        for i, block in enumerate(plan.layers):
+            if isinstance(block.ffn, RoutedExpertsSpec):
+                share[f"l{i}.mlp.e"] = 1.0 - (1.0 - block.ffn.top / block.ffn.n_experts) ** batch
+        total = 0.0
+        for name, decl in expected_tensors(plan).items():
+            if name in ("embed", "side.embed"):
+                continue
+            n = 1
+            for s in decl.shape:
+                n *= max(s, 1)
+            total += n * next((f for p, f in share.items() if name.startswith(p)), 1.0)
+        return int(total * item)
+
     def step_cache_bytes(self, batch: int, context: int, item: int) -> int:
         """Bytes of cache and state that a decode step of ``batch`` requests behind ``context`` tokens reads."""
         total = 0

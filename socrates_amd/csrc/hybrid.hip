@@ -535,12 +535,160 @@ grouped_linear_kernel(const T* __restrict__ x, int ldx, const int* __restrict__ 
         }
 }
 
-// x [*, K]; w [E, 2 ff or n_out, K]; out [M, n_out] in the compute dtype (out_f32 0) or float32 (1).
+// The same products in bfloat16 on the matrix cores. A workgroup of four waves (WM x WN) takes a tile of
+// BM = WM * MI * 16 places of one expert and BN = WN * NI * 16 weight rows, 64 k at a time through LDS, each wave
+// MI x NI products of 16 x 16 x 32 with float32 sums; the places' rows of x are gathered while they are staged.
+// With GLU a wave's weight tiles alternate between gate rows and the up rows of the same columns, so the
+// activation is taken in registers and a workgroup writes BN / 2 columns of it.
+typedef __attribute__((ext_vector_type(8))) __bf16 hyb_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float hyb_f32x4;
+constexpr int GM_BK = 64, GM_STRIDE = GM_BK + 8;
+
+template <int WM, int WN, int MI, int NI, bool GLU, typename TO>
+__global__ void __launch_bounds__(256)
+grouped_mfma_kernel(const bf16* __restrict__ x, int ldx, const int* __restrict__ pair_at, int top, const bf16* __restrict__ w,
+                    const int* __restrict__ offsets, const int* __restrict__ tiles, TO* __restrict__ out, int n_out, int K, int ff,
+                    float limit, float slope) {
+    constexpr int BM = WM * MI * 16, BN = WN * NI * 16, COLS = GLU ? BN / 2 : BN;
+    constexpr int A_PER = (BM * 8 + 255) / 256, W_PER = BN * 8 / 256;
+    static_assert(WM * WN == 4 && (!GLU || NI % 2 == 0), "four waves; gate and up tiles in pairs");
+    __shared__ __attribute__((aligned(16))) uint16_t As[BM * GM_STRIDE];
+    __shared__ __attribute__((aligned(16))) uint16_t Ws[BN * GM_STRIDE];
+    __shared__ int rows[BM];
+    const int e = tiles[2 * blockIdx.y];
+    if (e < 0) return;
+    const int p0 = tiles[2 * blockIdx.y + 1], pend = offsets[e + 1];
+    const int o0 = blockIdx.x * COLS;
+    const int tid = threadIdx.x, wave = tid / SOC_WAVE, lane = tid % SOC_WAVE;
+    const int wm = wave / WN, wn = wave % WN, li = lane % 16, lk = (lane / 16) * 8;
+    for (int i = tid; i < BM; i += 256) {
+        const int p = p0 + i;
+        rows[i] = p < pend ? (pair_at ? pair_at[p] / top : p) : -1;
+    }
+    __syncthreads();
+    const int w_rows = GLU ? 2 * ff : n_out;
+    const bf16* we = w + (size_t)e * w_rows * K;
+    // the weight row behind row r of the LDS tile (-1: none)
+    auto weight_row = [&](int r) {
+        if (!GLU) return o0 + r < n_out ? o0 + r : -1;
+        const int rw = r / (NI * 16), j = (r % (NI * 16)) / 16, col = o0 + rw * (NI / 2 * 16) + (j / 2) * 16 + r % 16;
+        return col < ff ? col + (j % 2 ? ff : 0) : -1;
+    };
+    const bf16* a_src[A_PER];
+    const bf16* w_src[W_PER];
+#pragma unroll
+    for (int i = 0; i < A_PER; ++i) {
+        const int c = tid + 256 * i, r = c < BM * 8 ? rows[c / 8] : -1;
+        a_src[i] = r >= 0 ? x + (size_t)r * ldx + (c % 8) * 8 : nullptr;
+    }
+#pragma unroll
+    for (int i = 0; i < W_PER; ++i) {
+        const int c = tid + 256 * i, r = weight_row(c / 8);
+        w_src[i] = r >= 0 ? we + (size_t)r * K + (c % 8) * 8 : nullptr;
+    }
+    hyb_f32x4 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = (hyb_f32x4){0.f, 0.f, 0.f, 0.f};
+    uint4 ra[A_PER], rw[W_PER];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < A_PER; ++i) {
+            const int kc = ((tid + 256 * i) % 8) * 8;
+            ra[i] = (a_src[i] && k0 + kc < K) ? *reinterpret_cast<const uint4*>(a_src[i] + k0) : make_uint4(0u, 0u, 0u, 0u);
+        }
+#pragma unroll
+        for (int i = 0; i < W_PER; ++i) {
+            const int kc = ((tid + 256 * i) % 8) * 8;
+            rw[i] = (w_src[i] && k0 + kc < K) ? *reinterpret_cast<const uint4*>(w_src[i] + k0) : make_uint4(0u, 0u, 0u, 0u);
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int i = 0; i < A_PER; ++i) {
+            const int c = tid + 256 * i;
+            if (c < BM * 8) *reinterpret_cast<uint4*>(&As[(c / 8) * GM_STRIDE + (c % 8) * 8]) = ra[i];
+        }
+#pragma unroll
+        for (int i = 0; i < W_PER; ++i) {
+            const int c = tid + 256 * i;
+            *reinterpret_cast<uint4*>(&Ws[(c / 8) * GM_STRIDE + (c % 8) * 8]) = rw[i];
+        }
+    };
+    fetch(0);
+    stash();
+    __syncthreads();
+    for (int k0 = 0; k0 < K; k0 += GM_BK) {
+        const bool more = k0 + GM_BK < K;
+        if (more) fetch(k0 + GM_BK);
+#pragma unroll
+        for (int ks = 0; ks < GM_BK; ks += 32) {
+            hyb_bf16x8 af[MI], wf[NI];
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+                af[i] = *reinterpret_cast<const hyb_bf16x8*>(&As[((wm * MI + i) * 16 + li) * GM_STRIDE + ks + lk]);
+#pragma unroll
+            for (int j = 0; j < NI; ++j)
+                wf[j] = *reinterpret_cast<const hyb_bf16x8*>(&Ws[((wn * NI + j) * 16 + li) * GM_STRIDE + ks + lk]);
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+        if (more) { stash(); __syncthreads(); }
+    }
+    // acc[i][j][r] belongs to place row 4 * (lane / 16) + r of tile i and weight row lane % 16 of tile j
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int p = p0 + (wm * MI + i) * 16 + (lane / 16) * 4 + r;
+            if (p >= pend) continue;
+            if constexpr (GLU) {
+#pragma unroll
+                for (int j = 0; j < NI; j += 2) {
+                    const int col = o0 + wn * (NI / 2 * 16) + (j / 2) * 16 + li;
+                    if (col >= ff) continue;
+                    const float g = fminf(to_float(from_float<bf16>(acc[i][j][r])), limit);
+                    const float u = fminf(fmaxf(to_float(from_float<bf16>(acc[i][j + 1][r])), -limit), limit);
+                    out[(size_t)p * n_out + col] = from_float<TO>(g * hyb_sigmoid(slope * g) * (u + 1.f));
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NI; ++j) {
+                    const int col = o0 + (wn * NI + j) * 16 + li;
+                    if (col < n_out) out[(size_t)p * n_out + col] = from_float<TO>(acc[i][j][r]);
+                }
+            }
+        }
+}
+
+// x [*, K]; w [E, 2 ff or n_out, K]; out [M, n_out] in the compute dtype (out_f32 0) or float32 (1). tile: the
+// places per tile that the sorting kernel was given: 16 (any dtype; bfloat16 with K and ldx multiples of 8 on the
+// matrix cores) or 128 (bfloat16 on the matrix cores only).
 SOC_EXPORT int soc_grouped_linear(const void* x, int ldx, const int* pair_at, int top, const void* w, const int* offsets,
-                                  const int* tiles, int max_tiles, void* out, int n_out, int K, int ff, float limit, float slope,
-                                  int out_f32, int dtype, hipStream_t stream) {
+                                  const int* tiles, int max_tiles, int tile, void* out, int n_out, int K, int ff, float limit,
+                                  float slope, int out_f32, int dtype, hipStream_t stream) {
     if (max_tiles <= 0 || n_out <= 0) return 0;
     if (K < 1 || max_tiles > 65535 || (ff > 0 && (ff != n_out || out_f32))) return (int)hipErrorInvalidValue;
+    const bool mfma = dtype == 1 && K % 8 == 0 && ldx % 8 == 0;
+    if ((tile != 16 && tile != 128) || (tile == 128 && !mfma)) return (int)hipErrorInvalidValue;
+    if (mfma) {
+#define SOC_GM(WM, WN, MI, NI, GLU, TO)                                                                                          \
+    hipLaunchKernelGGL((grouped_mfma_kernel<WM, WN, MI, NI, GLU, TO>), dim3((n_out + (GLU ? 63 : 127)) / (GLU ? 64 : 128), max_tiles), \
+                       dim3(256), 0, stream, (const bf16*)x, ldx, pair_at, top, (const bf16*)w, offsets, tiles, (TO*)out, n_out, \
+                       K, ff, limit, slope)
+        if (tile == 128) {
+            if (ff > 0) SOC_GM(2, 2, 4, 4, true, bf16); else if (out_f32) SOC_GM(2, 2, 4, 4, false, float); else SOC_GM(2, 2, 4, 4, false, bf16);
+        } else {
+            if (ff > 0) SOC_GM(1, 4, 1, 2, true, bf16); else if (out_f32) SOC_GM(1, 4, 1, 2, false, float); else SOC_GM(1, 4, 1, 2, false, bf16);
+        }
+#undef SOC_GM
+        return soc_last_error();
+    }
     const dim3 grid((n_out + 63) / 64, max_tiles);
 #define SOC_GL(T, TO, GLU)                                                                                                    \
     hipLaunchKernelGGL((grouped_linear_kernel<T, TO, GLU>), grid, dim3(256), 0, stream, (const T*)x, ldx, pair_at, top,       \

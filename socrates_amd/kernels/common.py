@@ -72,7 +72,7 @@ _HYBRID_SIGNATURES = {
     "soc_relu_squared": [P, P, L, I, P],
     "soc_moe_route": [P, P, I, I, I, I, I, F, P, P, P],
     "soc_moe_sort": [P, I, I, I, I, P, P, P, P, P],
-    "soc_grouped_linear": [P, I, P, I, P, P, P, I, P, I, I, I, F, F, I, I, P],
+    "soc_grouped_linear": [P, I, P, I, P, P, P, I, I, P, I, I, I, F, F, I, I, P],
     "soc_moe_combine": [P, P, P, P, P, I, I, I, I, P],
     "soc_side_gate": [P, P, I, I, P, I, P, I, I, I, P],
     "soc_add_cast": [P, P, P, I, L, P, I, P],

@@ -13,17 +13,19 @@ from .build import load_library
 from .common import _HYBRID_SIGNATURES, KernelError, _check, _declare, _ptr
 
 MAX_EXPERTS = 256        # what the routing and sorting kernels hold per token and per workgroup
-EXPERT_TILE = 16         # places of one expert that a workgroup of the products per expert takes
+EXPERT_TILE = 16         # places of one expert that a workgroup of the products per expert takes ...
+EXPERT_TILE_MANY = 128   # ... or, in bfloat16, where an expert has many tokens
+EXPERT_MANY = 48         # tokens per expert, on average, from which the larger tile is taken
 
 
 class ExpertRuns:
     """Tokens sorted by expert: ``place`` [M] (where each (token, choice) pair lies), ``pair_at`` [M] (which
     pair lies at a place), ``offsets`` [E + 1] (each expert's run of places) and ``tiles`` [max_tiles, 2]
     ((expert, first place) of every tile the products walk; expert -1 behind the last)."""
-    __slots__ = ("place", "pair_at", "offsets", "tiles", "top")
+    __slots__ = ("place", "pair_at", "offsets", "tiles", "top", "tile")
 
-    def __init__(self, place, pair_at, offsets, tiles, top):
-        self.place, self.pair_at, self.offsets, self.tiles, self.top = place, pair_at, offsets, tiles, top
+    def __init__(self, place, pair_at, offsets, tiles, top, tile):
+        self.place, self.pair_at, self.offsets, self.tiles, self.top, self.tile = place, pair_at, offsets, tiles, top, tile
 
 
 class Hybrid:
@@ -154,20 +156,23 @@ class Hybrid:
                "moe_route")
         return idx, weight
 
-    def moe_sort(self, idx, E):
-        """The (token, choice) pairs of ``idx`` [N, top] laid out expert by expert: an ``ExpertRuns``."""
+    def moe_sort(self, idx, E, tile=EXPERT_TILE):
+        """The (token, choice) pairs of ``idx`` [N, top] laid out expert by expert, in tiles of ``tile`` places: an
+        ``ExpertRuns``."""
         N, top = idx.shape
         self._want(idx, "experts", torch.int32)
         if not 1 <= E <= MAX_EXPERTS:
             raise KernelError(f"{E} experts (at most {MAX_EXPERTS})")
+        if tile not in (EXPERT_TILE, EXPERT_TILE_MANY):
+            raise KernelError(f"tiles of {tile} places")
         M = N * top
-        max_tiles = (M + EXPERT_TILE - 1) // EXPERT_TILE + min(E, M)
+        max_tiles = (M + tile - 1) // tile + min(E, M)
         ints = torch.empty((2 * M + E + 1 + 2 * max_tiles,), dtype=torch.int32, device=self.device)
         place, pair_at, offsets = ints[:M], ints[M:2 * M], ints[2 * M:2 * M + E + 1]
         tiles = ints[2 * M + E + 1:].view(max_tiles, 2)
-        _check(self._hybrid().soc_moe_sort(_ptr(idx), c_int(M), c_int(E), c_int(EXPERT_TILE), c_int(max_tiles), _ptr(offsets),
+        _check(self._hybrid().soc_moe_sort(_ptr(idx), c_int(M), c_int(E), c_int(tile), c_int(max_tiles), _ptr(offsets),
                                            _ptr(place), _ptr(pair_at), _ptr(tiles), self._stream()), "moe_sort")
-        return ExpertRuns(place, pair_at, offsets, tiles, top)
+        return ExpertRuns(place, pair_at, offsets, tiles, top, tile)
 
     def grouped_linear(self, x, w, runs, by_token, glu=None, out_dtype=None):
         """out[p] = w[e] x[row of p] for every place p of expert e's run; x rows are tokens (``by_token``: place p
@@ -192,7 +197,7 @@ class Hybrid:
         limit, slope = glu if glu is not None else (0.0, 0.0)
         _check(self._hybrid().soc_grouped_linear(
             _ptr(x), c_int(x.stride(0)), _ptr(runs.pair_at if by_token else None), c_int(runs.top), _ptr(w), _ptr(runs.offsets),
-            _ptr(runs.tiles), c_int(runs.tiles.shape[0]), _ptr(out), c_int(n_out), c_int(K), c_int(ff), c_float(limit),
+            _ptr(runs.tiles), c_int(runs.tiles.shape[0]), c_int(runs.tile), _ptr(out), c_int(n_out), c_int(K), c_int(ff), c_float(limit),
             c_float(slope), c_int(1 if out_dtype == torch.float32 and self.dtype != torch.float32 else 0), c_int(self.code),
             self._stream()), "grouped_linear")
         return out
@@ -218,7 +223,12 @@ class Hybrid:
     def moe_experts(self, x, idx, weight, w_gate_up, w_down, limit, slope, extra=None):
         """The weighted sum of each token's chosen experts (clamped gated feed-forwards: ``w_gate_up`` [E, 2 ff, d],
         ``w_down`` [E, d, ff]) plus ``extra``; float32 [N, d]."""
-        runs = self.moe_sort(idx, w_gate_up.shape[0])
+        E, _, d = w_gate_up.shape
+        ff = w_down.shape[2]
+        # many tokens per expert, in bfloat16 with rows that start on 16 bytes: the larger tile of the matrix cores
+        many = (self.dtype == torch.bfloat16 and idx.numel() >= EXPERT_MANY * E and d % 8 == 0 and ff % 8 == 0
+                and x.stride(0) % 8 == 0)
+        runs = self.moe_sort(idx, E, EXPERT_TILE_MANY if many else EXPERT_TILE)
         act = self.grouped_linear(x, w_gate_up, runs, by_token=True, glu=(limit, slope))
         y = self.grouped_linear(act, w_down, runs, by_token=False, out_dtype=torch.float32)
         return self.moe_combine(y, runs, weight, extra)
