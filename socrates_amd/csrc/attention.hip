@@ -1115,7 +1115,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                           int table_width, const int* __restrict__ token_rows,
                           const int* __restrict__ positions, const int* __restrict__ row_blocks,
                           bf16* __restrict__ out, int Hq, int Hkv, int BS, int bs_shift, float scale,
-                          int window, int group_pad_log2) {
+                          int window, int group_pad_log2, int keep_first, int sink) {
     static_assert(D <= 128, "one key pair per thread");
     static_assert(KS == 1 || (KS == 2 && M32), "key halves come with the 32-row products");
     constexpr int PF_TILE_ELEMS = PF_K_ELEMS + PF_V_ELEMS;          // one K tile and one V^T tile
@@ -1137,8 +1137,17 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     const int tokens_per_wave = ((M32 ? 32 : 16 * RT)) >> group_pad_log2;
 
     const int khi = pos0 + ntok;                                    // keys any row of the block sees
-    const int kmin = window > 0 ? max(0, pos0 - window + 1) : 0;
+    int kmin = window > 0 ? max(0, pos0 - window + 1) : 0;
+    // With a window, the keys below keep_first stay visible. Those of them that lie before the window of the
+    // block's first row (kept of them) are walked first, in tiles of their own that stand in front of the
+    // window's tiles (n_pre of them, the walk then starts at the virtual key klo - n_pre * PF_KEYS); where
+    // such tiles would reach into the window's, the walk starts at key 0 instead and the mask does the rest.
+    int kept = window > 0 ? min(keep_first, kmin) : 0, n_pre = (kept + PF_KEYS - 1) / PF_KEYS;
+    if (n_pre * PF_KEYS > (kmin & ~(PF_KEYS - 1))) { kmin = 0; kept = 0; n_pre = 0; }
     int klo = kmin & ~(PF_KEYS - 1);
+    const int first_real = klo;                                     // virtual keys from here on are real ones
+    const int pre_shift = klo - n_pre * PF_KEYS;                    // a virtual key before that is the real key minus this
+    if (KS == 1) klo = pre_shift;
     // kend: where this half's walk over the tiles ends. Both halves take the same number of
     // steps (they share the barriers); the second may run past khi, where keys are stand-ins
     // that no row sees.
@@ -1216,13 +1225,13 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     auto lookup = [&](int key0, int (&pg)[2]) {
         if constexpr (PAIR) {
             const int key = key0 + 2 * kp;
-            const bool ok = key + 1 >= kmin && key < khi;
+            const bool ok = (key + 1 >= kmin || key < kept) && key < khi;
             pg[0] = pg[1] = table[ok ? key >> bs_shift : 0];
         } else {
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const int key = key0 + 2 * kp + h;
-                const bool ok = key >= kmin && key < khi;
+                const bool ok = (key >= kmin || key < kept) && key < khi;
                 pg[h] = table[ok ? (bs_shift >= 0 ? key >> bs_shift : key / BS) : 0];
             }
         }
@@ -1250,8 +1259,8 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         uint4 k0 = kr[0], k1 = kr[1], v0 = vr[0], v1 = vr[1];
         if (key0 < kmin || key0 + PF_KEYS > khi) {           // uniform: a tile at an edge of the range
             const int key = key0 + 2 * kp;
-            if (key < kmin || key >= khi) { k0 = make_uint4(0u, 0u, 0u, 0u); v0 = k0; }
-            if (key + 1 < kmin || key + 1 >= khi) { k1 = make_uint4(0u, 0u, 0u, 0u); v1 = k1; }
+            if ((key < kmin && key >= kept) || key >= khi) { k0 = make_uint4(0u, 0u, 0u, 0u); v0 = k0; }
+            if ((key + 1 < kmin && key + 1 >= kept) || key + 1 >= khi) { k1 = make_uint4(0u, 0u, 0u, 0u); v1 = k1; }
         }
         const int r0 = M32 ? pf_k_row32(2 * kp) : pf_k_row(2 * kp), r1 = M32 ? pf_k_row32(2 * kp + 1) : pf_k_row(2 * kp + 1);
         *reinterpret_cast<uint4*>(&k_lds[buf][r0 * PF_K_STRIDE + part * 8]) = k0;
@@ -1298,7 +1307,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                 if constexpr (MASKED) {
                     const int key = key0 + 8 * kb + r;
                     bool seen = key <= row_pos[rt];
-                    if (window > 0) seen = seen && key > row_pos[rt] - window;
+                    if (window > 0) seen = seen && (key > row_pos[rt] - window || key < keep_first);
                     t[r] = seen ? t[r] : -INFINITY;
                 }
                 mx = fmaxf(mx, t[r]);
@@ -1364,7 +1373,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
             if constexpr (MASKED) {
                 const int key = key0 + 16 * (i / 8) + 8 * g32 + i % 8;
                 bool seen = key <= row_pos32;
-                if (window > 0) seen = seen && key > row_pos32 - window;
+                if (window > 0) seen = seen && (key > row_pos32 - window || key < keep_first);
                 sc[i] = seen ? sc[i] : -INFINITY;
             }
             mx = fmaxf(mx, sc[i]);
@@ -1453,42 +1462,45 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     };
     int pg0[2], pg1[2];
     uint4 kr0[2], vr0[2], kr1[2], vr1[2];
-    lookup(klo, pg0);
-    lookup(klo + PF_KEYS, pg1);
-    fetch(klo, pg0, kr0, vr0);
-    lookup(klo + 2 * PF_KEYS, pg0);
-    if (klo + PF_KEYS < kend) fetch(klo + PF_KEYS, pg1, kr1, vr1);
-    stash(0, klo, kr0, vr0);
+    // (the walk is over virtual keys: the tiles of the kept first keys stand in front of the window's)
+    auto real = [&](int v) { return v < first_real ? v - pre_shift : v; };
+    lookup(real(klo), pg0);
+    lookup(real(klo + PF_KEYS), pg1);
+    fetch(real(klo), pg0, kr0, vr0);
+    lookup(real(klo + 2 * PF_KEYS), pg0);
+    if (klo + PF_KEYS < kend) fetch(real(klo + PF_KEYS), pg1, kr1, vr1);
+    stash(0, real(klo), kr0, vr0);
     __syncthreads();
     int key0 = klo;
     for (; key0 + 3 * PF_KEYS < kend; key0 += 2 * PF_KEYS) {
-        lookup(key0 + 3 * PF_KEYS, pg1);
-        fetch(key0 + 2 * PF_KEYS, pg0, kr0, vr0);
-        tile(key0, 0);
-        stash(1, key0 + PF_KEYS, kr1, vr1);
+        lookup(real(key0 + 3 * PF_KEYS), pg1);
+        fetch(real(key0 + 2 * PF_KEYS), pg0, kr0, vr0);
+        tile(real(key0), 0);
+        stash(1, real(key0 + PF_KEYS), kr1, vr1);
         __syncthreads();
-        lookup(key0 + 4 * PF_KEYS, pg0);
-        fetch(key0 + 3 * PF_KEYS, pg1, kr1, vr1);
-        tile(key0 + PF_KEYS, 1);
-        stash(0, key0 + 2 * PF_KEYS, kr0, vr0);
+        lookup(real(key0 + 4 * PF_KEYS), pg0);
+        fetch(real(key0 + 3 * PF_KEYS), pg1, kr1, vr1);
+        tile(real(key0 + PF_KEYS), 1);
+        stash(0, real(key0 + 2 * PF_KEYS), kr0, vr0);
         __syncthreads();
     }
     const bool has1 = key0 + PF_KEYS < kend, has2 = key0 + 2 * PF_KEYS < kend;    // the same in all threads
-    if (has2) fetch(key0 + 2 * PF_KEYS, pg0, kr0, vr0);
-    tile(key0, 0);
+    if (has2) fetch(real(key0 + 2 * PF_KEYS), pg0, kr0, vr0);
+    tile(real(key0), 0);
     if (has1) {
-        stash(1, key0 + PF_KEYS, kr1, vr1);
+        stash(1, real(key0 + PF_KEYS), kr1, vr1);
         __syncthreads();
-        tile(key0 + PF_KEYS, 1);
+        tile(real(key0 + PF_KEYS), 1);
         if (has2) {
-            stash(0, key0 + 2 * PF_KEYS, kr0, vr0);
+            stash(0, real(key0 + 2 * PF_KEYS), kr0, vr0);
             __syncthreads();
-            tile(key0 + 2 * PF_KEYS, 0);
+            tile(real(key0 + 2 * PF_KEYS), 0);
         }
     }
 
     if constexpr (M32) {
         float L = sum_xor32(l32);
+        float m_ref = m32 == -INFINITY ? 0.f : m32;          // what the weights in L are relative to
         if constexpr (KS == 2) {
             // the second half hands its result over: [wave][value][lane] floats where the tiles were
             static_assert(KS * 2 * PF_TILE_ELEMS * 2 >= 4 * 64 * (16 * DB32 + 2) * 4, "the tiles' space holds the exchange");
@@ -1509,11 +1521,13 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
             const float ms = mn == -INFINITY ? 0.f : mn;
             const float wa = __builtin_amdgcn_exp2f(m32 - ms), wb = __builtin_amdgcn_exp2f(m_b - ms);
             L = L * wa + l_b * wb;
+            m_ref = ms;
 #pragma unroll
             for (int b = 0; b < DB32; ++b)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) o32[b][i] = o32[b][i] * wa + xch[(16 * b + i) * 64] * wb;
         }
+        if (sink) L += __builtin_amdgcn_exp2f(-m_ref);       // one more weight of score 0, no value
         if (row_pos32 >= 0) {
             const float inv = L > 0.f ? 1.0f / L : 0.f;
 #pragma unroll
@@ -1533,6 +1547,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         float L = l[rt];
         L = sum_xor32(sum_xor16(L));
         if (row_pos[rt] < 0) continue;
+        if (sink) L += __builtin_amdgcn_exp2f(-(m[rt] == -INFINITY ? 0.f : m[rt]));   // one more weight of score 0, no value
         const float inv = L > 0.f ? 1.0f / L : 0.f;
 #pragma unroll
         for (int j = 0; j < DV; ++j) {
@@ -1548,15 +1563,18 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
 // token, tokens) of each block of at most 4 * ((16 * row_tiles) >> group_pad_log2) tokens of
 // one sequence, or null: every token is a block of its own. row_tiles 32: a wave owns 32 rows
 // (blocks of at most 4 * (32 >> group_pad_log2) tokens), head sizes that are multiples of 32;
-// row_tiles 64: the same with eight waves, four for each half of a block's keys.
+// row_tiles 64: the same with eight waves, four for each half of a block's keys. keep_first (with a window): the
+// keys below it stay visible to every row (not with row_tiles 64); sink: one more weight of score 0 and no value
+// in every row's sum.
 SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, const void* v_pool,
                                            const int* block_table, int table_width, const int* token_rows,
                                            const int* positions, const int* row_blocks, int n_row_blocks,
                                            void* out, int N, int Hq, int Hkv, int BS, float scale,
-                                           int window, int row_tiles, int group_pad_log2,
+                                           int window, int row_tiles, int group_pad_log2, int keep_first, int sink,
                                            hipStream_t stream) {
     if (N <= 0 || n_row_blocks <= 0) return 0;
-    if (Hkv < 1 || Hq % Hkv || BS < 1) return (int)hipErrorInvalidValue;
+    if (Hkv < 1 || Hq % Hkv || BS < 1 || keep_first < 0) return (int)hipErrorInvalidValue;
+    if (row_tiles == 64 && (keep_first > 0 && window > 0)) return (int)hipErrorInvalidValue;   // no kept keys with key halves
     if (!(scale > 0.f)) return (int)hipErrorInvalidValue;        // the maximum is taken of the raw scores
     if (!row_blocks && n_row_blocks != N) return (int)hipErrorInvalidValue;
     const int G = Hq / Hkv;
@@ -1568,7 +1586,8 @@ SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, co
         for (bs_shift = 0; (1 << bs_shift) < BS; ++bs_shift) {}
     if constexpr (D <= 128) {
 #define SOC_PF_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
-        token_rows, positions, row_blocks, (bf16*)out, Hq, Hkv, BS, bs_shift, scale, window, group_pad_log2
+        token_rows, positions, row_blocks, (bf16*)out, Hq, Hkv, BS, bs_shift, scale, window, group_pad_log2, \
+        keep_first, sink
         const bool pair = bs_shift >= 1;
 #define SOC_PF_LAUNCH(RT_, M32_, KS_)                                                                            \
     do {                                                                                                    \

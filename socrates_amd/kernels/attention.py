@@ -293,7 +293,7 @@ class Attention:
         G = Hq // Hkv
         softcap, sinks, slopes, keep_first = 0.0, None, None, 0
         if terms:
-            known = {"softcap", "sinks", "slopes", "keep_first"}
+            known = {"softcap", "sinks", "slopes", "keep_first", "zero_sink"}
             if set(terms) - known:
                 raise KernelError(f"attention: unknown score terms {sorted(set(terms) - known)}")
             softcap = float(terms.get("softcap") or 0.0)
@@ -307,7 +307,14 @@ class Attention:
                 if t is not None:
                     self._want(t, name, torch.float32, (Hq,))
         plain = softcap == 0.0 and sinks is None and slopes is None and scale > 0 and keep_first == 0
-        if self.dtype == torch.bfloat16 and self.attention_mfma and plain:
+        # The kernel that shares K and V tiles among four waves also takes kept first keys and an added weight of
+        # score 0 (``sinks`` all zero: ``terms["zero_sink"]`` says so without a look at the device); the per-wave
+        # kernel with key splits does not, so a step with a long portion sends all its rows to the former (behind
+        # a window no row walks far), and steps of short portions and decoded tokens go to the vector-unit kernel.
+        zero_sink = bool(terms and terms.get("zero_sink")) and sinks is not None
+        windowed = (softcap == 0.0 and slopes is None and scale > 0 and (sinks is None or zero_sink)
+                    and (keep_first > 0 or zero_sink))
+        if self.dtype == torch.bfloat16 and self.attention_mfma and (plain or windowed):
             gpl = max(0, (min(G, 16) - 1).bit_length())
             decode = getattr(ctx, "max_q_len", 1) == 1
             if N > 65535:
@@ -318,7 +325,7 @@ class Attention:
             # kernel it would hold four waves and walk its whole context alone).
             lens = self._portion_lengths(ctx)
             long_ = None if lens is None else lens >= self.SHORT_PORTION
-            mixed = not decode and long_ is not None and bool(long_.any()) and not bool(long_.all())
+            mixed = not decode and long_ is not None and bool(long_.any()) and not bool(long_.all()) and not windowed
             n_long = int(lens[long_].sum()) if mixed else N
             # Row tiles of the workgroup kernel. 1, 2: 16 or 32 rows per wave through the
             # 16 x 16 products; 32: 32 rows per wave through the 32 x 32 products (head sizes
@@ -342,7 +349,7 @@ class Attention:
                 if n32 >= th["four_waves_of_32_rows"] and D > 64:
                     wg_rt = 32
                 elif n32 >= th["eight_waves"]:
-                    wg_rt = 64
+                    wg_rt = 64 if not keep_first else 32      # (no kept keys with the keys in two halves)
             elif D <= 64 and (n_long // (4 * max(1, 32 >> gpl))) * Hkv * ((G + 15) // 16) >= th["two_tiles_of_16_rows"]:
                 wg_rt = 2
             wg_tokens = 4 * max(1, (32 if wg_rt >= 32 else 16 * wg_rt) >> gpl)
@@ -354,6 +361,8 @@ class Attention:
             # the row tiles (tests) forces the choice.
             enough = ((n_long // wg_tokens) * Hkv * ((G + 15) // 16) >= th["workgroup_kernel"]
                       or self.attention_row_tiles is not None)
+            if keep_first and wg_rt == 64:
+                wg_rt = 32
             if (self.attention_workgroup and not decode and D <= 128 and self.attention_splits is None
                     and getattr(ctx, "max_q_len", 1) >= 16 and enough):
                 rt = wg_rt
@@ -363,18 +372,20 @@ class Attention:
                     _ptr(q), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
                     c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(blocks),
                     c_int(n_blocks), _ptr(out), c_int(N), c_int(Hq), c_int(Hkv), c_int(slot.block_size),
-                    c_float(scale), c_int(w), c_int(rt), c_int(gpl), self._stream()),
-                    "paged_attention (prefill)")
+                    c_float(scale), c_int(w), c_int(rt), c_int(gpl), c_int(keep_first), c_int(1 if zero_sink else 0),
+                    self._stream()), "paged_attention (prefill)")
                 if mixed:
                     # after the long ones, on the same stream: side by side on a second stream
                     # was measured and is slower (35.4 ms against 32.3 ms per mixed step at 8B sizes)
                     self._wave_attention(lib, q, slot, ctx, out, scale, w, 1, gpl, "short")
                 return out
-            rt = self.attention_row_tiles or 1
-            rt = min(rt, 4 if D <= 64 else (2 if D <= 128 else 1))      # what the kernel is built with
-            self.last_attention_kernel = ("wave", rt)
-            self._wave_attention(lib, q, slot, ctx, out, scale, w, rt, gpl, None)
-            return out
+            if not windowed:
+                rt = self.attention_row_tiles or 1
+                rt = min(rt, 4 if D <= 64 else (2 if D <= 128 else 1))      # what the kernel is built with
+                self.last_attention_kernel = ("wave", rt)
+                self._wave_attention(lib, q, slot, ctx, out, scale, w, rt, gpl, None)
+                return out
+        self.last_attention_kernel = ("tokens", 0)
         max_keys = ctx.max_ctx_len if not w else min(w + keep_first, ctx.max_ctx_len)
         split_len, n_splits = self.plan_splits(N, Hkv, G, max_keys)
         part_o = part_ml = None

@@ -63,6 +63,7 @@ class GatedWindowAttention:
         terms = {}
         if spec.sink:
             terms["sinks"] = torch.zeros(H, dtype=torch.float32, device=ops.device)
+            terms["zero_sink"] = True            # (all of them zero: said here, so that nobody has to look)
         if spec.window is not None and spec.keep_first:
             terms["keep_first"] = spec.keep_first
         self.terms = terms or None

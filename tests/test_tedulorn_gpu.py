@@ -147,6 +147,40 @@ def test_attention_keeps_the_first_keys(kernel_sets, dtype, window, keep):
         assert not torch.allclose(other.float(), want.float(), atol=0.05)
 
 
+@pytest.mark.parametrize("row_tiles", [None, 1, 2, 32])
+@pytest.mark.parametrize("window,keep,P,G", [(40, 7, 32, 2), (100, 33, 64, 1), (64, 64, 128, 4), (7, 100, 48, 2), (500, 3, 64, 2), (33, 0, 32, 1)])
+def test_prompt_attention_on_the_matrix_cores_keeps_the_first_keys(kernel_sets, window, keep, P, G, row_tiles):
+    """Long portions go to the kernel that shares its key tiles among four waves: kept first keys in tiles of their
+    own in front of the window's, the added weight, rows of several sequences (one from position 0, one behind 300
+    cached tokens, single tokens beside them), every form of the kernel, against the stand-in."""
+    from socrates_amd.cache.manager import PagedSlot
+    ops, dt = kernel_sets["bfloat16"], torch.bfloat16
+    if row_tiles == 32 and P % 32:
+        pytest.skip("32-row products take head sizes in steps of 32")
+    ref = TorchKernels(dt, DEV)
+    g = torch.Generator(device="cpu").manual_seed(window + keep)
+    Hkv, bs = 2, 16
+    Hq = Hkv * G
+    lengths, rows, starts = [700, 1, 230, 1, 17], [0, 1, 2, 3, 4], [0, 59, 300, 5, 140]
+    ctx = _ctx(lengths, rows, starts, DEV)
+    pages = 48
+    table = torch.arange(1, 1 + 5 * pages, dtype=torch.int32, device=DEV).view(5, pages)
+    table = torch.cat([table, torch.zeros(1, pages, dtype=torch.int32, device=DEV)]).contiguous()
+    slot = PagedSlot((torch.randn(1 + 5 * pages, Hkv, bs, P, generator=g) * 0.8).to(dt).to(DEV),
+                     torch.randn(1 + 5 * pages, Hkv, bs, P, generator=g).to(dt).to(DEV), table, bs, window)
+    q = torch.randn(ctx.n_tokens, Hq, P, generator=g).to(dt).to(DEV)
+    terms = {"sinks": torch.zeros(Hq, dtype=torch.float32, device=DEV), "keep_first": keep, "zero_sink": True}
+    want = ref.paged_attention(q, slot, ctx, 0.3, window, terms=terms)
+    ops.attention_row_tiles = row_tiles
+    try:
+        got = ops.paged_attention(q, slot, ctx, 0.3, window, terms=terms)
+        kernel = ops.last_attention_kernel
+    finally:
+        ops.attention_row_tiles = None
+    assert kernel[0] == ("workgroup" if row_tiles else kernel[0])
+    _close(got, want, "bfloat16", f"window {window}, {keep} kept, row tiles {row_tiles} ({kernel})")
+
+
 @pytest.mark.parametrize("E,top,count,keep", [(12, 3, 4, 2), (6, 2, 3, 1), (8, 8, 2, 2), (5, 1, 5, 2), (9, 4, 1, 1), (256, 8, 8, 4), (70, 6, 1, 1)])
 def test_the_choice_of_experts_kernel(kernel_sets, E, top, count, keep):
     ops, ref = kernel_sets["float32"], TorchKernels(torch.float32, DEV)
