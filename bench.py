@@ -334,7 +334,7 @@ def tedulorn_beside_others(args, dtype, item):
            "sizes": {}}
     only = set(filter(None, (args.only or "").split(",")))
     for tag, preset, heads in sizes:
-        if only and tag not in only:
+        if only & {name for name, _, _ in sizes} and tag not in only:
             continue
         q = preset_dict(preset)
         q["num_hidden_layers"] = n_layers

@@ -555,6 +555,9 @@ grouped_mfma_kernel(const bf16* __restrict__ x, int ldx, const int* __restrict__
     __shared__ __attribute__((aligned(16))) uint16_t As[BM * GM_STRIDE];
     __shared__ __attribute__((aligned(16))) uint16_t Ws[BN * GM_STRIDE];
     __shared__ int rows[BM];
+    // (columns along x: workgroups that start together share a tile's rows of x. Measured the other way round,
+    // tiles along x so that an expert's tiles share weight rows, a prompt of 2,048 tokens at 4B-sized layers took
+    // 24.8 instead of 22.4 ms.)
     const int e = tiles[2 * blockIdx.y];
     if (e < 0) return;
     const int p0 = tiles[2 * blockIdx.y + 1], pend = offsets[e + 1];
@@ -668,20 +671,22 @@ grouped_mfma_kernel(const bf16* __restrict__ x, int ldx, const int* __restrict__
 
 // x [*, K]; w [E, 2 ff or n_out, K]; out [M, n_out] in the compute dtype (out_f32 0) or float32 (1). tile: the
 // places per tile that the sorting kernel was given: 16 (any dtype; bfloat16 with K and ldx multiples of 8 on the
-// matrix cores) or 128 (bfloat16 on the matrix cores only).
+// matrix cores) or 128 or 256 (bfloat16 on the matrix cores only).
 SOC_EXPORT int soc_grouped_linear(const void* x, int ldx, const int* pair_at, int top, const void* w, const int* offsets,
                                   const int* tiles, int max_tiles, int tile, void* out, int n_out, int K, int ff, float limit,
                                   float slope, int out_f32, int dtype, hipStream_t stream) {
     if (max_tiles <= 0 || n_out <= 0) return 0;
     if (K < 1 || max_tiles > 65535 || (ff > 0 && (ff != n_out || out_f32))) return (int)hipErrorInvalidValue;
     const bool mfma = dtype == 1 && K % 8 == 0 && ldx % 8 == 0;
-    if ((tile != 16 && tile != 128) || (tile == 128 && !mfma)) return (int)hipErrorInvalidValue;
+    if ((tile != 16 && tile != 128 && tile != 256) || (tile > 16 && !mfma)) return (int)hipErrorInvalidValue;
     if (mfma) {
 #define SOC_GM(WM, WN, MI, NI, GLU, TO)                                                                                          \
     hipLaunchKernelGGL((grouped_mfma_kernel<WM, WN, MI, NI, GLU, TO>), dim3((n_out + (GLU ? 63 : 127)) / (GLU ? 64 : 128), max_tiles), \
                        dim3(256), 0, stream, (const bf16*)x, ldx, pair_at, top, (const bf16*)w, offsets, tiles, (TO*)out, n_out, \
                        K, ff, limit, slope)
-        if (tile == 128) {
+        if (tile == 256) {
+            if (ff > 0) SOC_GM(2, 2, 8, 4, true, bf16); else if (out_f32) SOC_GM(2, 2, 8, 4, false, float); else SOC_GM(2, 2, 8, 4, false, bf16);
+        } else if (tile == 128) {
             if (ff > 0) SOC_GM(2, 2, 4, 4, true, bf16); else if (out_f32) SOC_GM(2, 2, 4, 4, false, float); else SOC_GM(2, 2, 4, 4, false, bf16);
         } else {
             if (ff > 0) SOC_GM(1, 4, 1, 2, true, bf16); else if (out_f32) SOC_GM(1, 4, 1, 2, false, float); else SOC_GM(1, 4, 1, 2, false, bf16);

@@ -14,8 +14,10 @@ from .common import _HYBRID_SIGNATURES, KernelError, _check, _declare, _ptr
 
 MAX_EXPERTS = 256        # what the routing and sorting kernels hold per token and per workgroup
 EXPERT_TILE = 16         # places of one expert that a workgroup of the products per expert takes ...
-EXPERT_TILE_MANY = 128   # ... or, in bfloat16, where an expert has many tokens
-EXPERT_MANY = 48         # tokens per expert, on average, from which the larger tile is taken
+# ... or, in bfloat16, (tokens per expert on average from which, places). Tiles of 256 from 160 tokens per expert on
+# were measured and lost (a prompt of 2,048 tokens at 4B-sized layers, 256 tokens per expert on average: 25.1 against
+# 22.4 ms: half the experts then need a second tile that is nearly empty).
+EXPERT_TILES_MANY = ((1024, 256), (48, 128))
 
 
 class ExpertRuns:
@@ -163,7 +165,7 @@ class Hybrid:
         self._want(idx, "experts", torch.int32)
         if not 1 <= E <= MAX_EXPERTS:
             raise KernelError(f"{E} experts (at most {MAX_EXPERTS})")
-        if tile not in (EXPERT_TILE, EXPERT_TILE_MANY):
+        if tile not in (EXPERT_TILE,) + tuple(t for _, t in EXPERT_TILES_MANY):
             raise KernelError(f"tiles of {tile} places")
         M = N * top
         max_tiles = (M + tile - 1) // tile + min(E, M)
@@ -225,10 +227,12 @@ class Hybrid:
         ``w_down`` [E, d, ff]) plus ``extra``; float32 [N, d]."""
         E, _, d = w_gate_up.shape
         ff = w_down.shape[2]
-        # many tokens per expert, in bfloat16 with rows that start on 16 bytes: the larger tile of the matrix cores
-        many = (self.dtype == torch.bfloat16 and idx.numel() >= EXPERT_MANY * E and d % 8 == 0 and ff % 8 == 0
-                and x.stride(0) % 8 == 0)
-        runs = self.moe_sort(idx, E, EXPERT_TILE_MANY if many else EXPERT_TILE)
+        # many tokens per expert, in bfloat16 with rows that start on 16 bytes: the larger tiles of the matrix cores
+        # (a weight row then comes from memory once per 128 or 256 tokens of its expert)
+        tile = EXPERT_TILE
+        if self.dtype == torch.bfloat16 and d % 8 == 0 and ff % 8 == 0 and x.stride(0) % 8 == 0:
+            tile = next((t for least, t in EXPERT_TILES_MANY if idx.numel() >= least * E), EXPERT_TILE)
+        runs = self.moe_sort(idx, E, tile)
         act = self.grouped_linear(x, w_gate_up, runs, by_token=True, glu=(limit, slope))
         y = self.grouped_linear(act, w_down, runs, by_token=False, out_dtype=torch.float32)
         return self.moe_combine(y, runs, weight, extra)

@@ -196,7 +196,7 @@ def test_the_choice_of_experts_kernel(kernel_sets, E, top, count, keep):
 
 @pytest.mark.parametrize("dtype", list(DTYPES))
 @pytest.mark.parametrize("N,E,top,d,ff", [(1, 4, 1, 24, 8), (7, 6, 2, 40, 20), (50, 12, 3, 64, 24), (300, 5, 5, 72, 100), (129, 33, 4, 128, 48),
-                                         (600, 4, 2, 64, 40), (2000, 6, 3, 256, 136)])
+                                         (600, 4, 2, 64, 40), (2000, 6, 3, 256, 136), (300, 8, 2, 64, 48)])
 def test_routed_experts_kernels(kernel_sets, dtype, N, E, top, d, ff):
     """Sorting by expert, the two products per expert and the weighted sum against the stand-in, which runs
     every token's experts one by one; experts that nobody chose and experts with more than one tile of tokens."""
