@@ -150,14 +150,46 @@ SOC_EXPORT int soc_head_gate(const void* o, const void* g, int ldg, void* out, i
 // ---- retention: S <- decay S + k v^T, o = S^T q, a fixed decay per head -------------------------------------
 // x: rows of ld elements with H heads of D (q, from col_q; k, from col_k) and H heads of Dv (v, from col_v).
 // q and k are turned over their first 2 * half elements by the token's position and k is scaled, in float32,
-// while a batch of tokens is staged. The state [H, D, Dv] of the sequence's row is float32; a workgroup owns
-// CW columns of one head, thread (part, column) a slice of the keys. o goes out in float32 [N, H * Dv].
+// while a batch of tokens is staged, or ahead of the walk by a kernel of its own (turned: [N, 2, H * D] float32;
+// every workgroup of a head's columns would turn the head's q and k again, which costs a long portion more than
+// the walk itself). The state [H, D, Dv] of the sequence's row is float32; a workgroup owns CW columns of one
+// head, thread (part, column) a slice of the keys. o goes out in float32 [N, H * Dv].
+// q and k of every token turned by its position over their first 2 * half elements and k scaled, float32:
+// turned [N, 2, H * D]. One thread per (token, head, pair) and per element behind the turned part.
+template <typename T>
+__global__ void retention_turn_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, const int* __restrict__ positions,
+                                      const float* __restrict__ inv_freq, int half, float k_scale, int H, int D, size_t total,
+                                      float* __restrict__ turned) {
+    const int per = half + (D - 2 * half);                 // work items of one head: pairs, then single elements
+    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
+        const int w = (int)(e % per);
+        const size_t nh = e / per;
+        const int h = (int)(nh % H);
+        const size_t n = nh / H;
+        const T* row = x + n * ld + h * D;
+        float* q = turned + n * 2 * H * D + (size_t)h * D;
+        float* k = q + (size_t)H * D;
+        if (w < half) {
+            const float a = to_float(row[col_q + w]), b = to_float(row[col_q + w + half]);
+            const float a2 = to_float(row[col_k + w]), b2 = to_float(row[col_k + w + half]);
+            float sn, cs;
+            sincosf((float)positions[n] * inv_freq[w], &sn, &cs);
+            q[w] = a * cs - b * sn; q[w + half] = b * cs + a * sn;
+            k[w] = (a2 * cs - b2 * sn) * k_scale; k[w + half] = (b2 * cs + a2 * sn) * k_scale;
+        } else {
+            const int d = 2 * half + (w - half);
+            q[d] = to_float(row[col_q + d]);
+            k[d] = to_float(row[col_k + d]) * k_scale;
+        }
+    }
+}
+
 template <typename T, int DK, int CW>
 __global__ void __launch_bounds__(256)
 retention_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, int col_v, const int* __restrict__ positions,
                  const float* __restrict__ inv_freq, int half, float k_scale, const float* __restrict__ decays, int H, int D,
                  int Dv, float* __restrict__ state, size_t stride, int offset, const int* __restrict__ seq_qstart,
-                 const int* __restrict__ seq_rows, float* __restrict__ out) {
+                 const int* __restrict__ seq_rows, const float* __restrict__ turned, float* __restrict__ out) {
     constexpr int REC_TB = rec_batch(DK), PARTS = 256 / CW, KPT = DK / PARTS, STAGE = (REC_TB * DK + 255) / 256;
     __shared__ float sq[2][REC_TB][DK], sk[2][REC_TB][DK];
     __shared__ float red[REC_TB][PARTS][CW];
@@ -181,7 +213,11 @@ retention_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, int col_
             const int e = tid + q * 256, t = e / DK, i = e % DK;
             const bool in = t < REC_TB && n0 + t < hi && i < D;
             float a = 0.f, b = 0.f;
-            if (in) {
+            if (in && turned) {                        // q and k were turned and scaled ahead, [N, 2, H * D] float32
+                const float* row = turned + (size_t)(n0 + t) * 2 * H * D + head * D + i;
+                a = row[0];
+                b = row[(size_t)H * D];
+            } else if (in) {
                 const T* row = x + (size_t)(n0 + t) * ld + head * D;
                 a = to_float(row[col_q + i]);
                 b = to_float(row[col_k + i]);
@@ -255,25 +291,35 @@ retention_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, int col_
 template <typename T, int DK>
 static void launch_retention(const void* x, int ld, int col_q, int col_k, int col_v, const int* positions, const float* inv_freq,
                              int half, float k_scale, const float* decays, int H, int D, int Dv, float* state, long long stride,
-                             int offset, const int* seq_qstart, const int* seq_rows, float* out, int n_seqs, int cw,
-                             hipStream_t stream) {
+                             int offset, const int* seq_qstart, const int* seq_rows, const float* turned, float* out, int n_seqs,
+                             int cw, hipStream_t stream) {
 #define SOC_RET_LAUNCH(CW)                                                                                                     \
     hipLaunchKernelGGL((retention_kernel<T, DK, CW>), dim3(H * ((Dv + CW - 1) / CW), n_seqs), dim3(256), 0, stream,            \
                        (const T*)x, ld, col_q, col_k, col_v, positions, inv_freq, half, k_scale, decays, H, D, Dv, state,      \
-                       (size_t)stride, offset, seq_qstart, seq_rows, out)
+                       (size_t)stride, offset, seq_qstart, seq_rows, turned, out)
     if (cw == 16) SOC_RET_LAUNCH(16); else SOC_RET_LAUNCH(64);
 #undef SOC_RET_LAUNCH
 }
 
 SOC_EXPORT int soc_retention(const void* x, int ld, int col_q, int col_k, int col_v, const int* positions, const float* inv_freq,
                              int half, float k_scale, const float* decays, int H, int D, int Dv, float* state, long long stride,
-                             int offset, const int* seq_qstart, const int* seq_rows, float* out, int n_seqs, int max_q_len,
-                             int dtype, hipStream_t stream) {
+                             int offset, const int* seq_qstart, const int* seq_rows, float* turned, int n_tokens, float* out,
+                             int n_seqs, int max_q_len, int dtype, hipStream_t stream) {
     if (n_seqs <= 0 || H <= 0) return 0;
     if (D < 1 || D > 256 || Dv < 1 || n_seqs > 65535 || 2 * half > D) return (int)hipErrorInvalidValue;
+    if (turned) {                                          // scratch [n_tokens, 2, H * D]: turn q and k ahead of the walk
+        const size_t total = (size_t)n_tokens * H * (D - half);
+        const int blocks = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
+        if (dtype == 0)
+            hipLaunchKernelGGL(retention_turn_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)x, ld, col_q, col_k,
+                               positions, inv_freq, half, k_scale, H, D, total, turned);
+        else
+            hipLaunchKernelGGL(retention_turn_kernel<bf16>, dim3(blocks), dim3(256), 0, stream, (const bf16*)x, ld, col_q, col_k,
+                               positions, inv_freq, half, k_scale, H, D, total, turned);
+    }
     const int cw = columns_per_workgroup(H, Dv, n_seqs, max_q_len);
-#define SOC_RET_F32(DK) launch_retention<float, DK>(x, ld, col_q, col_k, col_v, positions, inv_freq, half, k_scale, decays, H, D, Dv, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, cw, stream)
-#define SOC_RET_BF16(DK) launch_retention<bf16, DK>(x, ld, col_q, col_k, col_v, positions, inv_freq, half, k_scale, decays, H, D, Dv, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, cw, stream)
+#define SOC_RET_F32(DK) launch_retention<float, DK>(x, ld, col_q, col_k, col_v, positions, inv_freq, half, k_scale, decays, H, D, Dv, state, stride, offset, seq_qstart, seq_rows, turned, out, n_seqs, cw, stream)
+#define SOC_RET_BF16(DK) launch_retention<bf16, DK>(x, ld, col_q, col_k, col_v, positions, inv_freq, half, k_scale, decays, H, D, Dv, state, stride, offset, seq_qstart, seq_rows, turned, out, n_seqs, cw, stream)
     if (dtype == 0) { SOC_BY_STATE_SIZE(D, SOC_RET_F32) } else { SOC_BY_STATE_SIZE(D, SOC_RET_BF16) }
     return soc_last_error();
 }
@@ -552,8 +598,8 @@ grouped_mfma_kernel(const bf16* __restrict__ x, int ldx, const int* __restrict__
     constexpr int BM = WM * MI * 16, BN = WN * NI * 16, COLS = GLU ? BN / 2 : BN;
     constexpr int A_PER = (BM * 8 + 255) / 256, W_PER = BN * 8 / 256;
     static_assert(WM * WN == 4 && (!GLU || NI % 2 == 0), "four waves; gate and up tiles in pairs");
-    __shared__ __attribute__((aligned(16))) uint16_t As[BM * GM_STRIDE];
-    __shared__ __attribute__((aligned(16))) uint16_t Ws[BN * GM_STRIDE];
+    __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * GM_STRIDE];     // two buffers: one barrier per 64 k
+    __shared__ __attribute__((aligned(16))) uint16_t Ws[2][BN * GM_STRIDE];
     __shared__ int rows[BM];
     // (columns along x: workgroups that start together share a tile's rows of x. Measured the other way round,
     // tiles along x so that an expert's tiles share weight rows, a prompt of 2,048 tokens at 4B-sized layers took
@@ -607,41 +653,46 @@ grouped_mfma_kernel(const bf16* __restrict__ x, int ldx, const int* __restrict__
             rw[i] = (w_src[i] && k0 + kc < K) ? *reinterpret_cast<const uint4*>(w_src[i] + k0) : make_uint4(0u, 0u, 0u, 0u);
         }
     };
-    auto stash = [&]() {
+    auto stash = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < A_PER; ++i) {
             const int c = tid + 256 * i;
-            if (c < BM * 8) *reinterpret_cast<uint4*>(&As[(c / 8) * GM_STRIDE + (c % 8) * 8]) = ra[i];
+            if (c < BM * 8) *reinterpret_cast<uint4*>(&As[buf][(c / 8) * GM_STRIDE + (c % 8) * 8]) = ra[i];
         }
 #pragma unroll
         for (int i = 0; i < W_PER; ++i) {
             const int c = tid + 256 * i;
-            *reinterpret_cast<uint4*>(&Ws[(c / 8) * GM_STRIDE + (c % 8) * 8]) = rw[i];
+            *reinterpret_cast<uint4*>(&Ws[buf][(c / 8) * GM_STRIDE + (c % 8) * 8]) = rw[i];
         }
     };
+    // blocks of 16 places of this wave that hold a place at all (the last tile of an expert is seldom full)
+    const int n_sub = min(MI, max(0, (pend - p0 - wm * MI * 16 + 15) / 16));
     fetch(0);
-    stash();
+    stash(0);
     __syncthreads();
-    for (int k0 = 0; k0 < K; k0 += GM_BK) {
+    int buf = 0;
+    for (int k0 = 0; k0 < K; k0 += GM_BK, buf ^= 1) {
         const bool more = k0 + GM_BK < K;
         if (more) fetch(k0 + GM_BK);
 #pragma unroll
         for (int ks = 0; ks < GM_BK; ks += 32) {
-            hyb_bf16x8 af[MI], wf[NI];
-#pragma unroll
-            for (int i = 0; i < MI; ++i)
-                af[i] = *reinterpret_cast<const hyb_bf16x8*>(&As[((wm * MI + i) * 16 + li) * GM_STRIDE + ks + lk]);
+            hyb_bf16x8 wf[NI];
 #pragma unroll
             for (int j = 0; j < NI; ++j)
-                wf[j] = *reinterpret_cast<const hyb_bf16x8*>(&Ws[((wn * NI + j) * 16 + li) * GM_STRIDE + ks + lk]);
+                wf[j] = *reinterpret_cast<const hyb_bf16x8*>(&Ws[buf][((wn * NI + j) * 16 + li) * GM_STRIDE + ks + lk]);
 #pragma unroll
-            for (int i = 0; i < MI; ++i)
+            for (int i = 0; i < MI; ++i) {
+                if (i < n_sub) {                              // the same in all lanes of the wave
+                    const hyb_bf16x8 af = *reinterpret_cast<const hyb_bf16x8*>(&As[buf][((wm * MI + i) * 16 + li) * GM_STRIDE + ks + lk]);
 #pragma unroll
-                for (int j = 0; j < NI; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+                    for (int j = 0; j < NI; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, wf[j], acc[i][j], 0, 0, 0);
+                }
+            }
         }
+        // the other buffer was last read before the barrier that ended the previous round
+        if (more) stash(buf ^ 1);
         __syncthreads();
-        if (more) { stash(); __syncthreads(); }
     }
     // acc[i][j][r] belongs to place row 4 * (lane / 16) + r of tile i and weight row lane % 16 of tile j
 #pragma unroll
@@ -671,22 +722,20 @@ grouped_mfma_kernel(const bf16* __restrict__ x, int ldx, const int* __restrict__
 
 // x [*, K]; w [E, 2 ff or n_out, K]; out [M, n_out] in the compute dtype (out_f32 0) or float32 (1). tile: the
 // places per tile that the sorting kernel was given: 16 (any dtype; bfloat16 with K and ldx multiples of 8 on the
-// matrix cores) or 128 or 256 (bfloat16 on the matrix cores only).
+// matrix cores) or 128 (bfloat16 on the matrix cores only).
 SOC_EXPORT int soc_grouped_linear(const void* x, int ldx, const int* pair_at, int top, const void* w, const int* offsets,
                                   const int* tiles, int max_tiles, int tile, void* out, int n_out, int K, int ff, float limit,
                                   float slope, int out_f32, int dtype, hipStream_t stream) {
     if (max_tiles <= 0 || n_out <= 0) return 0;
     if (K < 1 || max_tiles > 65535 || (ff > 0 && (ff != n_out || out_f32))) return (int)hipErrorInvalidValue;
     const bool mfma = dtype == 1 && K % 8 == 0 && ldx % 8 == 0;
-    if ((tile != 16 && tile != 128 && tile != 256) || (tile > 16 && !mfma)) return (int)hipErrorInvalidValue;
+    if ((tile != 16 && tile != 128) || (tile > 16 && !mfma)) return (int)hipErrorInvalidValue;
     if (mfma) {
 #define SOC_GM(WM, WN, MI, NI, GLU, TO)                                                                                          \
     hipLaunchKernelGGL((grouped_mfma_kernel<WM, WN, MI, NI, GLU, TO>), dim3((n_out + (GLU ? 63 : 127)) / (GLU ? 64 : 128), max_tiles), \
                        dim3(256), 0, stream, (const bf16*)x, ldx, pair_at, top, (const bf16*)w, offsets, tiles, (TO*)out, n_out, \
                        K, ff, limit, slope)
-        if (tile == 256) {
-            if (ff > 0) SOC_GM(2, 2, 8, 4, true, bf16); else if (out_f32) SOC_GM(2, 2, 8, 4, false, float); else SOC_GM(2, 2, 8, 4, false, bf16);
-        } else if (tile == 128) {
+        if (tile == 128) {
             if (ff > 0) SOC_GM(2, 2, 4, 4, true, bf16); else if (out_f32) SOC_GM(2, 2, 4, 4, false, float); else SOC_GM(2, 2, 4, 4, false, bf16);
         } else {
             if (ff > 0) SOC_GM(1, 4, 1, 2, true, bf16); else if (out_f32) SOC_GM(1, 4, 1, 2, false, float); else SOC_GM(1, 4, 1, 2, false, bf16);

@@ -68,7 +68,7 @@ _MIXER_SIGNATURES = {
 _HYBRID_SIGNATURES = {
     "soc_attn_prepare": [P, I, I, I, I, P, I, P, P, P, P, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, P],
     "soc_head_gate": [P, P, I, P, I, I, I, I, I, P],
-    "soc_retention": [P, I, I, I, I, P, P, I, F, P, I, I, I, P, L, I, P, P, P, I, I, I, P],
+    "soc_retention": [P, I, I, I, I, P, P, I, F, P, I, I, I, P, L, I, P, P, P, I, P, I, I, I, P],
     "soc_relu_squared": [P, P, L, I, P],
     "soc_moe_route": [P, P, I, I, I, I, I, F, P, P, P],
     "soc_moe_sort": [P, I, I, I, I, P, P, P, P, P],

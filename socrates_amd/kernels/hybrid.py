@@ -14,10 +14,9 @@ from .common import _HYBRID_SIGNATURES, KernelError, _check, _declare, _ptr
 
 MAX_EXPERTS = 256        # what the routing and sorting kernels hold per token and per workgroup
 EXPERT_TILE = 16         # places of one expert that a workgroup of the products per expert takes ...
-# ... or, in bfloat16, (tokens per expert on average from which, places). Tiles of 256 from 160 tokens per expert on
-# were measured and lost (a prompt of 2,048 tokens at 4B-sized layers, 256 tokens per expert on average: 25.1 against
-# 22.4 ms: half the experts then need a second tile that is nearly empty).
-EXPERT_TILES_MANY = ((1024, 256), (48, 128))
+# ... or, in bfloat16, (tokens per expert on average from which, places). Tiles of 256 places were measured and lost
+# (a prompt of 2,048 tokens at 4B-sized layers, 256 tokens per expert on average: 20.5 against 17.6 ms).
+EXPERT_TILES_MANY = ((48, 128),)
 
 
 class ExpertRuns:
@@ -31,6 +30,8 @@ class ExpertRuns:
 
 
 class Hybrid:
+    retention_turn_ahead = 16       # tokens of a step's longest portion from which q and k are turned ahead of the walk
+
     def _hybrid(self):
         lib = getattr(self, "_hybrid_lib", None)
         if lib is None:
@@ -125,11 +126,16 @@ class Hybrid:
         self._want(decays, "decays", torch.float32, (H,))
         stride = self._state(state, offset, H * D * Dv, ctx)
         out = torch.empty((N, H * Dv), dtype=torch.float32, device=self.device)
+        # a step with a portion of some length: q and k are turned once, ahead of the walk (each of a head's
+        # workgroups would turn them again); single tokens and short portions are turned where they are staged
+        turned = None
+        if half and ctx.max_q_len >= self.retention_turn_ahead:
+            turned = torch.empty((N, 2, H * D), dtype=torch.float32, device=self.device)
         _check(self._hybrid().soc_retention(
             _ptr(x), c_int(ld), c_int(col_q), c_int(col_k), c_int(col_v), _ptr(ctx.positions), _ptr(inv_freq if half else None),
             c_int(half), c_float(k_scale), _ptr(decays), c_int(H), c_int(D), c_int(Dv), _ptr(state), stride, c_int(offset),
-            _ptr(ctx.seq_qstart), _ptr(ctx.seq_rows), _ptr(out), c_int(ctx.n_seqs), c_int(ctx.max_q_len), c_int(self.code),
-            self._stream()), "retention")
+            _ptr(ctx.seq_qstart), _ptr(ctx.seq_rows), _ptr(turned), c_int(N), _ptr(out), c_int(ctx.n_seqs), c_int(ctx.max_q_len),
+            c_int(self.code), self._stream()), "retention")
         return out
 
     # -- feed-forwards --------------------------------------------------------------------------------------------

@@ -81,7 +81,7 @@ def drawn_model(seed):
     multiples of anything (and sometimes 1), windows of one token up to longer than the prompts, kept first tokens
     from none to more than the window, groups of one expert and one group of all, layers without feed-forward."""
     rng = random.Random(seed)
-    width = rng.choice([24, 40, 56, 64, 88, 128])
+    width = rng.choice([24, 36, 40, 50, 56, 64, 88, 128])
     layers, mlps = [], []
     blended = None
     for _ in range(rng.randint(2, 5)):

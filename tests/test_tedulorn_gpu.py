@@ -60,11 +60,14 @@ def _ctx(lengths, rows, starts, dev):
 # ---- each kernel against its stand-in ----------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", list(DTYPES))
 @pytest.mark.parametrize("H,D,Dv,rot", [(3, 20, 28, 12), (1, 48, 80, 48), (4, 8, 8, 0), (2, 64, 40, 32), (2, 128, 64, 64), (1, 200, 16, 6)])
-def test_retention_kernel(kernel_sets, dtype, H, D, Dv, rot):
+@pytest.mark.parametrize("lengths", [[9, 1, 2, 15], [37, 1, 2, 170]])
+def test_retention_kernel(kernel_sets, dtype, H, D, Dv, rot, lengths):
+    """Steps of short portions (q and k turned where they are staged) and a step with a long one (turned ahead of
+    the walk), from a state that is not zero, several sequences of unequal length side by side."""
     ops, dt = kernel_sets[dtype], DTYPES[dtype]
     ref = TorchKernels(dt, DEV)
     g = torch.Generator(device="cpu").manual_seed(H * D + Dv)
-    lengths, rows, starts = [37, 1, 2, 70], [2, 0, 3, 1], [5, 300, 0, 41]
+    rows, starts = [2, 0, 3, 1], [5, 300, 0, 41]
     ctx = _ctx(lengths, rows, starts, DEV)
     N, ld = ctx.n_tokens, 7 + H * (2 * D + 2 * Dv)
     x = (torch.randn(N, ld, generator=g) * 0.7).to(dt).to(DEV)
